@@ -1,0 +1,242 @@
+/*
+ * libspotlight_hip.so -- C ABI of the gfx950 (MI355X) decode-time retrieval
+ * path of Spotlight Attention.
+ *
+ * Plain pointers and sizes only; every pointer is DEVICE memory unless said
+ * otherwise.  The library never allocates, frees or synchronises: the caller
+ * owns every buffer (workspaces included) and every call only enqueues
+ * kernels on `stream` (a hipStream_t passed as void*, NULL = default stream).
+ * Every entry point returns SL_OK (0) or a negative sl_status; sl_strerror()
+ * turns it into text.  Calls are re-entrant as long as two calls in flight do
+ * not share a workspace.
+ *
+ * Citations name the reference interface each entry point replaces (paths
+ * relative to the reference checkout).
+ */
+#ifndef SPOTLIGHT_HIP_H
+#define SPOTLIGHT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    SL_OK = 0,
+    SL_ERR_NULL = -1,        /* required pointer is NULL                     */
+    SL_ERR_SHAPE = -2,       /* a size is <= 0, not divisible as required... */
+    SL_ERR_UNSUPPORTED = -3, /* shape/dtype outside what the kernels cover   */
+    SL_ERR_ALIGN = -4,       /* pointer or stride not aligned as required    */
+    SL_ERR_WORKSPACE = -5,   /* workspace missing or too small               */
+    SL_ERR_LAUNCH = -6       /* hipGetLastError() reported a launch failure  */
+} sl_status;
+
+typedef enum { SL_F32 = 0, SL_BF16 = 1, SL_F16 = 2 } sl_dtype;
+
+/* Which query heads are summed into the score of kv head h:
+ * INTERLEAVED q head g*KH + h  (attn_k4_q28.cu:38,75; attn_dx_u32.py:112)
+ * BLOCKED     q head h*G + g   (repeat_kv, spotlight_generation.py:128)     */
+typedef enum { SL_HEADMAP_INTERLEAVED = 0, SL_HEADMAP_BLOCKED = 1 } sl_head_map;
+
+const char *sl_strerror(int status);
+int sl_version(void);
+
+/* ---- (a) sign -> packed codes ------------------------------------------ */
+
+/* Replaces packbits() (spotlight/kernel/packbits.cu:28-63) and
+ * pack_dx_u32_func (spotlight/kernel/pack_dx_u32.py:35-59).
+ * out[i] bit j = (x[32 i + j] > 0); x holds 32*n_words contiguous elements of
+ * `dtype`; x must be 16-byte aligned. */
+int sl_pack_sign_u32(const void *x, int dtype, uint32_t *out, int64_t n_words, void *stream);
+
+/* Replaces pack_dx_u8_func (spotlight/kernel/pack_dx_u8.py:34-56).
+ * out[i] bit j = (x[8 i + j] > 0); any n_bytes >= 0. */
+int sl_pack_sign_u8(const void *x, int dtype, uint8_t *out, int64_t n_bytes, void *stream);
+
+/* ---- (a) fused hash MLP -> sign -> pack --------------------------------- */
+
+/* Replaces hash_fn + torch.sign (spotlight_generation.py:16-20,229-255;
+ * linearhashing_generation.py:224-231) followed by pack_cuda_func
+ * (spotlight/kernel/__init__.py:23) for the decode step's new vectors.
+ *   x      [B, H, d_in]            dtype
+ *   w1     [H, d_in, d_hid]        dtype      b1 [H, d_hid] or NULL
+ *   w2     [H, d_hid, nbits]       dtype      b2 [H, nbits] or NULL
+ *   codes  u32, element (b, h, w) at b*code_stride_b + h*code_stride_h + w
+ * n_layers == 1: codes = pack(x @ w1 + b1 (+ x)), d_hid is the code width
+ *                (w2, b2 ignored);
+ * n_layers == 2: codes = pack(h @ w2 + b2 (+ h)), h = silu(x @ w1 + b1) (+ x).
+ * `residue` adds the layer input to its output (needs equal widths).
+ * For bf16/f16 inputs every intermediate is rounded to that type exactly
+ * where the reference's torch expression rounds it; accumulation is fp32.
+ * code_row[b] (may be NULL, then 0) is added to the code row index, in units
+ * of code_stride_n, so that a key code lands in cache row seq_len[b].
+ * ws: sl_hash_workspace_bytes(B, H, d_hid, nbits) bytes, zeroed once with
+ * sl_workspace_init(); the kernel leaves it zeroed again. */
+size_t sl_hash_workspace_bytes(int B, int H, int d_hid, int nbits);
+int sl_hash_mlp_pack(const void *x, const void *w1, const void *b1, const void *w2,
+                     const void *b2, uint32_t *codes, int dtype, int n_layers, int B,
+                     int H, int d_in, int d_hid, int nbits, int residue,
+                     int64_t x_stride_b, int64_t code_stride_b, int64_t code_stride_h,
+                     int64_t code_stride_n, const int32_t *code_row, void *ws,
+                     size_t ws_bytes, void *stream);
+
+/* ---- (b) Hamming scorer -------------------------------------------------- */
+
+/* Replaces attn_k4_q28() (spotlight/kernel/attn_k4_q28.cu:100-138) and
+ * attn_dx_u32_func (spotlight/kernel/attn_dx_u32.py:131-161) for any
+ * QH = G*KH with KH dividing 256 and W in {1,2,4,8}.
+ *   q_code [B, QH, W] u32 (batch stride q_stride_b words)
+ *   k_code [B, n, KH, W] u32 token-major (batch stride k_stride_b words)
+ *   out    [B, n, KH] int16 (batch stride out_stride_b elements):
+ *          number of matching bits summed over the G query heads.
+ * seq_lens (may be NULL): per-batch token count on the device; rows at or
+ * beyond it are not read and their outputs are left untouched. */
+int sl_hamming_score(const uint32_t *q_code, const uint32_t *k_code, int16_t *out, int B,
+                     int64_t n, int KH, int G, int W, int64_t q_stride_b,
+                     int64_t k_stride_b, int64_t out_stride_b, int head_map,
+                     const int32_t *seq_lens, void *stream);
+
+/* Replaces attn_dx_u8_func (spotlight/kernel/attn_dx_u8.py:46-74).
+ * q [BH, D] u8, k [BH, n, D] u8 head-major, out [BH, n] u8 (wraps mod 256 as
+ * the reference's uint8 accumulator does).  D in {4, 8, 16, 32}. */
+int sl_hamming_score_u8(const uint8_t *q, const uint8_t *k, uint8_t *out, int BH, int64_t n,
+                        int D, void *stream);
+
+/* ---- (c) top-k by count-select ------------------------------------------ */
+
+/* Replaces attn.topk(k=budget, dim=1, sorted=False).indices
+ * (spotlight/modifiers/gpu_cache.py:50, cpu_cache.py:52-53).
+ *   score  int16, element (b, t, h) at b*stride_b + t*stride_n + h*stride_h,
+ *          0 <= score <= max_score <= 4607
+ *   idx    [B, KH, k] int32: the k largest scores of (b, h), ties to the
+ *          lowest token index, listed in ascending token order; when fewer
+ *          than k tokens exist the tail is filled with -1.
+ * seq_lens (may be NULL): per-batch token count on the device (<= n).
+ * ws: sl_topk_workspace_bytes(B, KH, max_score), zeroed once with
+ * sl_workspace_init(); left zeroed. */
+size_t sl_topk_workspace_bytes(int B, int KH, int max_score);
+int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                   int32_t *idx, int B, int64_t n, int KH, int k, int max_score,
+                   const int32_t *seq_lens, void *ws, size_t ws_bytes, void *stream);
+
+/* ---- gather --------------------------------------------------------------- */
+
+/* Replaces topk_and_gather's two torch.gather calls
+ * (spotlight/modifiers/gpu_cache.py:51-53).
+ *   keys, vals [B, L, KH, d] (batch stride kv_stride_b elements, row stride
+ *   KH*d) -> k_out, v_out [B, k, KH, d] contiguous; idx [B, KH, k] int32,
+ *   rows with idx < 0 are written as zeros.  d*elem_size multiple of 16. */
+int sl_gather_kv(const void *keys, const void *vals, const int32_t *idx, void *k_out, void *v_out,
+                 int dtype, int B, int KH, int d, int k, int64_t kv_stride_b, void *stream);
+
+/* ---- (d) cache append and LRU resident table ----------------------------- */
+
+/* Replaces the slice assignment of KVHash.update / KVCache.update
+ * (spotlight/modifiers/gpu_cache.py:38-45,108-118) with a device-side row
+ * index: for every b copies `t` rows of row_bytes bytes from src
+ * (b*src_stride_b bytes apart) to dst + b*dst_stride_b + (start + row[b]) *
+ * row_bytes, row[b] = seq_lens ? seq_lens[b] : 0.  row_bytes % 16 == 0. */
+int sl_cache_append(const void *src, void *dst, int B, int64_t t, int64_t row_bytes,
+                    int64_t src_stride_b, int64_t dst_stride_b, int64_t start,
+                    const int32_t *seq_lens, void *stream);
+
+/* LRU resident table; NO counterpart in the reference (its caches are
+ * append-only, gpu_cache.py:108-118; cpu_cache.py:105-130 re-fetches every
+ * selected row from host memory each step, which this table exists to avoid).
+ * One table of C slots per (b, kv head):
+ *   slot_token [B,KH,C] int32 (-1 empty), slot_stamp [B,KH,C] uint32 (0 never),
+ *   token_slot [B,KH,map_cap] int32 (-1 = not resident),
+ *   k_res, v_res [B,KH,C,d] resident rows.
+ * Step stamp + (stamp_dev ? *stamp_dev : 0), stamp_dev being an optional
+ * device word: wanted = idx[b,h,:k] U {new_token[b]}.  Resident wanted
+ * tokens are hits (stamp refreshed); the M others are misses and replace the
+ * M slots that are not hits and come first by (stamp, slot); misses in
+ * ascending token order pair with victims in ascending slot order; their K/V
+ * rows are copied from the full store keys/vals [B, L, KH, d].
+ * slots_out [B,KH,k] int32 receives the resident slot of every idx entry
+ * (-1 where idx is -1); stats [B,KH,2] uint32 accumulates (hits, misses).
+ * Requires k + 1 <= C <= 4096, idx ascending as sl_topk_select emits it. */
+int sl_lru_update(const int32_t *idx, const int32_t *new_token, int32_t *slot_token,
+                  uint32_t *slot_stamp, int32_t *token_slot, const void *keys, const void *vals,
+                  void *k_res, void *v_res, int32_t *slots_out, uint32_t *stats, int dtype, int B,
+                  int KH, int d, int k, int C, int64_t map_cap, int64_t kv_stride_b,
+                  uint32_t stamp, const uint32_t *stamp_dev, void *stream);
+
+/* ---- (e) sparse GQA decode attention -------------------------------------- */
+
+/* Replaces mask-scatter + do_sdpa_attn (spotlight_generation.py:200-215,
+ * modify_llama.py:151-186) and the intended flash_attn_func(q, K_sel, V_sel)
+ * (import at modify_llama.py:6) without materialising K_sel / V_sel.
+ *   q    [B, QH, d] dtype (batch stride q_stride_b elements)
+ *   keys, vals: row r of (b, h) at b*kv_stride_b + r*kv_stride_n + h*kv_stride_h
+ *               (elements), d contiguous elements
+ *   idx  [B, KH, k] int32 row numbers (negative entries are skipped)
+ *   out  [B, QH, d] dtype contiguous; kv head of q head qh is qh / G.
+ * d must be 128.  fp32 softmax and accumulation; scale <= 0 means 1/sqrt(d).
+ * ws: sl_attn_workspace_bytes(B, QH, KH, d, k), zeroed once; left zeroed. */
+size_t sl_attn_workspace_bytes(int B, int QH, int KH, int d, int k);
+int sl_sparse_gqa_attn(const void *q, const void *keys, const void *vals, const int32_t *idx,
+                       void *out, int dtype, int B, int QH, int KH, int d, int k,
+                       int64_t q_stride_b, int64_t kv_stride_b, int64_t kv_stride_n,
+                       int64_t kv_stride_h, float scale, void *ws, size_t ws_bytes,
+                       void *stream);
+
+/* ---- fused decode step ----------------------------------------------------- */
+
+/* One decode step of one layer: hash q and the new key, append code + K + V
+ * at row seq_lens[b], score all seq_lens[b]+1 codes, select the top k per
+ * (b, kv head), optional LRU update, attend over the selected rows, and
+ * finally seq_lens[b] += 1.  It is the composition the reference's kernel and
+ * cache layers are laid out for (attn_k4_q28.cu:118 -> gpu_cache.py:50-53 ->
+ * flash_attn_func) driven from self_attn_forward's decode branch
+ * (spotlight_generation.py:143-215). */
+typedef struct {
+    int dtype;              /* sl_dtype of q, k_new, v_new, K, V, weights, out   */
+    int B, QH, KH, d;       /* d == 128                                         */
+    int nbits;              /* code width in bits, multiple of 32 (W = nbits/32)*/
+    int k;                  /* tokens kept per (b, kv head)                     */
+    int head_map;           /* sl_head_map used by the scorer                   */
+    int64_t n_cap;          /* rows allocated per batch in codes / K / V        */
+    int64_t n_max;          /* upper bound of seq_lens[b] + 1 for this call     */
+    /* per-step inputs */
+    const void *q;          /* [B, QH, d]                                       */
+    const void *k_new;      /* [B, KH, d] post-RoPE                             */
+    const void *v_new;      /* [B, KH, d]                                       */
+    /* hash weights; n_layers in {1, 2}; *_k may alias *_q when KH == QH        */
+    int n_layers, d_hid, residue;
+    const void *w1_q, *b1_q, *w2_q, *b2_q;   /* [QH, ...]                       */
+    const void *w1_k, *b1_k, *w2_k, *b2_k;   /* [KH, ...]                       */
+    /* caches, token-major */
+    uint32_t *codes;        /* [B, n_cap, KH, W]                                */
+    void *keys, *vals;      /* [B, n_cap, KH, d]                                */
+    int32_t *seq_lens;      /* [B] tokens cached BEFORE this step; incremented  */
+    /* outputs */
+    void *out;              /* [B, QH, d]                                       */
+    int32_t *idx;           /* [B, KH, k] selected tokens, ascending            */
+    /* optional LRU resident table (lru_C == 0 disables it)                     */
+    int lru_C;
+    int64_t lru_map_cap;
+    int32_t *slot_token;
+    uint32_t *slot_stamp;
+    int32_t *token_slot;
+    void *k_res, *v_res;
+    int32_t *slots_out;     /* [B, KH, k]                                       */
+    uint32_t *lru_stats;    /* [B, KH, 2]                                       */
+    uint32_t *step_counter; /* [1] device counter, incremented every step       */
+    /* scratch */
+    void *ws;
+    size_t ws_bytes;
+} sl_decode_params;
+
+size_t sl_decode_workspace_bytes(const sl_decode_params *p);
+int sl_decode_step(const sl_decode_params *p, void *stream);
+
+/* Zero-fills a workspace with a kernel (safe inside a captured HIP graph). */
+int sl_workspace_init(void *ws, size_t ws_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPOTLIGHT_HIP_H */

@@ -1,0 +1,63 @@
+"""Builds libspotlight_hip.so for gfx950 with hipcc, in-tree.
+
+Run as ``python -m spotlight_amd.build``.  The library links against the HIP
+runtime only; there is no torch in it.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_NAME = "libspotlight_hip.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+
+SOURCES = ["pack.hip", "hamming.hip", "topk.hip", "attn.hip", "hash.hip", "cache.hip", "decode.hip"]
+
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; libspotlight_hip.so cannot be built")
+    return exe
+
+
+def build_library(verbose: bool = True, jobs: int = 4) -> str:
+    """Compile every kernel source and link the shared library.  Always
+    recompiles; returns the path of the built library."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    hipcc = _hipcc()
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_one(src: str) -> str:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(compile_one, SOURCES))
+    cmd = [hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library()
+    print(LIB_PATH)
+    sys.exit(0)

@@ -1,0 +1,178 @@
+// Shared device/host helpers for the gfx950 kernels.  wave64 throughout.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/spotlight_hip.h"
+
+#define SL_WAVE 64
+
+#define SL_REQUIRE(cond, code) \
+    do {                       \
+        if (!(cond)) return (code); \
+    } while (0)
+
+static inline int sl_check_launch() {
+    return hipGetLastError() == hipSuccess ? SL_OK : SL_ERR_LAUNCH;
+}
+
+static inline bool sl_aligned(const void *p, size_t a) {
+    return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+static inline size_t sl_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// ---- element types ---------------------------------------------------------
+// 16-bit floats travel as raw bits; arithmetic is always fp32.
+
+struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
+
+template <typename T> struct elem_traits;
+template <> struct elem_traits<float> { static constexpr int dtype = SL_F32; };
+template <> struct elem_traits<bf16_t> { static constexpr int dtype = SL_BF16; };
+template <> struct elem_traits<f16_t> { static constexpr int dtype = SL_F16; };
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// round-to-nearest-even, NaN kept quiet: the conversion torch applies.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(b)));
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return bf16_bits_to_f32(v.bits); }
+__device__ __forceinline__ float to_f32(f16_t v) { return f16_bits_to_f32(v.bits); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float f);
+template <> __device__ __forceinline__ float from_f32<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float f) {
+    return bf16_t{static_cast<uint16_t>(f32_to_bf16_bits(f))};
+}
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float f) {
+    return f16_t{static_cast<uint16_t>(f32_to_f16_bits(f))};
+}
+
+// value the reference's torch expression would hold after storing `f` in T
+template <typename T> __device__ __forceinline__ float round_to(float f) {
+    return to_f32(from_f32<T>(f));
+}
+
+// Unpack the two 16-bit halves of a 32-bit word to fp32.
+template <typename T> __device__ __forceinline__ void unpack2(uint32_t w, float &lo, float &hi);
+template <> __device__ __forceinline__ void unpack2<bf16_t>(uint32_t w, float &lo, float &hi) {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t w, float &lo, float &hi) {
+    lo = f16_bits_to_f32(w & 0xffffu);
+    hi = f16_bits_to_f32(w >> 16);
+}
+
+// Load 8 consecutive elements (16-byte aligned for 16-bit types, 32 for fp32)
+// as fp32.
+template <typename T> __device__ __forceinline__ void load8(const T *p, float (&v)[8]) {
+    if constexpr (sizeof(T) == 4) {
+        const float4 a = reinterpret_cast<const float4 *>(p)[0];
+        const float4 b = reinterpret_cast<const float4 *>(p)[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        const uint4 a = *reinterpret_cast<const uint4 *>(p);
+        unpack2<T>(a.x, v[0], v[1]);
+        unpack2<T>(a.y, v[2], v[3]);
+        unpack2<T>(a.z, v[4], v[5]);
+        unpack2<T>(a.w, v[6], v[7]);
+    }
+}
+
+// ---- wave64 cross-lane helpers ------------------------------------------------
+
+// DPP move; lanes whose source lies outside the row/wave, or whose row is
+// masked off, receive `identity`.
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf>
+__device__ __forceinline__ int dpp_i32(int identity, int v) {
+    return __builtin_amdgcn_update_dpp(identity, v, CTRL, ROW_MASK, BANK_MASK, false);
+}
+
+constexpr int DPP_QUAD_XOR1 = 0xB1;   // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;   // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_SHR1 = 0x111;
+constexpr int DPP_ROW_SHR2 = 0x112;
+constexpr int DPP_ROW_SHR4 = 0x114;
+constexpr int DPP_ROW_SHR8 = 0x118;
+constexpr int DPP_ROW_ROR4 = 0x124;
+constexpr int DPP_ROW_ROR8 = 0x128;
+constexpr int DPP_ROW_BCAST15 = 0x142;
+constexpr int DPP_ROW_BCAST31 = 0x143;
+
+// Sum over each aligned group of 16 lanes; every lane ends with the total.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(dpp_i32<DPP_QUAD_XOR1>(0, __float_as_int(v)));
+    v += __int_as_float(dpp_i32<DPP_QUAD_XOR2>(0, __float_as_int(v)));
+    v += __int_as_float(dpp_i32<DPP_ROW_ROR4>(0, __float_as_int(v)));
+    v += __int_as_float(dpp_i32<DPP_ROW_ROR8>(0, __float_as_int(v)));
+    return v;
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x) {
+    int v = static_cast<int>(x);
+    v += dpp_i32<DPP_ROW_SHR1>(0, v);
+    v += dpp_i32<DPP_ROW_SHR2>(0, v);
+    v += dpp_i32<DPP_ROW_SHR4>(0, v);
+    v += dpp_i32<DPP_ROW_SHR8>(0, v);
+    v += dpp_i32<DPP_ROW_BCAST15, 0xa>(0, v);  // lane 15 of rows 0/2 -> rows 1/3
+    v += dpp_i32<DPP_ROW_BCAST31, 0xc>(0, v);  // lane 31 -> rows 2,3
+    return static_cast<uint32_t>(v);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+
+// Exclusive prefix sum of one uint32 per thread over a block of NT threads
+// (NT multiple of 64, <= 1024).  `wave_tot` is NT/64 + 1 words of LDS.
+// Returns the exclusive prefix; *total receives the block sum.  Contains two
+// barriers; every thread of the block must call it.
+template <int NT>
+__device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t x, uint32_t *wave_tot,
+                                                        uint32_t *total) {
+    constexpr int NW = NT / 64;
+    const uint32_t inc = wave_inclusive_sum(x);
+    if (lane_id() == 63) wave_tot[wave_id()] = inc;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        uint32_t t = threadIdx.x < NW ? wave_tot[threadIdx.x] : 0u;
+        uint32_t ti = wave_inclusive_sum(t);
+        if (threadIdx.x < NW) wave_tot[threadIdx.x] = ti - t;
+        if (threadIdx.x == 63) wave_tot[NW] = ti;
+    }
+    __syncthreads();
+    const uint32_t base = wave_tot[wave_id()];
+    *total = wave_tot[NW];
+    return base + inc - x;
+}

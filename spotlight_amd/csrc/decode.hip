@@ -1,0 +1,171 @@
+// Fused decode step and the small library-level entry points.
+//
+// sl_decode_step enqueues, on one stream and without host synchronisation:
+//   1. hash_kernel       q codes -> workspace; new key's code, K and V -> cache row seq_lens[b]
+//   2. hamming_kernel    fused flavour: head-major scores + global histogram over seq_lens[b]+1 rows
+//   3. select_kernel     threshold from the histogram, stable compaction -> idx
+//   4. lru_kernel        (optional) resident-table update -> slot list
+//   5. sparse_attn_kernel over idx (or over the resident slots), then seq_lens[b] += 1
+// Every length is read from device memory, so the same captured HIP graph can
+// be replayed while the cache grows.
+#include "attn.h"
+#include "hamming.h"
+#include "hash.h"
+#include "lru.h"
+#include "topk.h"
+
+namespace {
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, uint8_t *tail, size_t n_tail) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (size_t j = i; j < n16; j += stride) p[j] = make_uint4(0, 0, 0, 0);
+    if (i < n_tail) tail[i] = 0;
+}
+
+struct ws_layout {
+    size_t q_code, hist, score, hash, attn, total;
+};
+
+ws_layout layout(const sl_decode_params &p) {
+    ws_layout L{};
+    const size_t W = static_cast<size_t>(p.nbits) / 32;
+    const size_t G = static_cast<size_t>(p.QH / p.KH);
+    size_t off = 0;
+    L.q_code = off; off += sl_align_up(sizeof(uint32_t) * p.B * p.QH * W, 256);
+    L.hist = off;   off += sl_align_up(sizeof(uint32_t) * p.B * p.KH * (G * p.nbits + 1), 256);
+    L.score = off;  off += sl_align_up(sizeof(int16_t) * p.B * p.KH * static_cast<size_t>(p.n_cap), 256);
+    L.hash = off;   off += sl_hash_ws_bytes(p.B, p.QH + p.KH, p.d_hid, p.nbits);
+    L.attn = off;   off += sl_attn_ws_bytes(p.B, p.QH, p.KH, p.k);
+    L.total = off;
+    return L;
+}
+
+int validate(const sl_decode_params &p) {
+    SL_REQUIRE(p.B > 0 && p.QH > 0 && p.KH > 0 && p.k > 0 && p.nbits > 0 && p.n_cap > 0 && p.n_max > 0, SL_ERR_SHAPE);
+    SL_REQUIRE(p.QH % p.KH == 0 && p.nbits % 32 == 0 && p.n_max <= p.n_cap, SL_ERR_SHAPE);
+    SL_REQUIRE(p.d == 128, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(p.n_cap % 8 == 0, SL_ERR_ALIGN);
+    SL_REQUIRE(HS_THREADS % p.KH == 0, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE((p.QH / p.KH) * p.nbits + 1 <= TK_MAX_BINS, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(p.q && p.k_new && p.v_new && p.codes && p.keys && p.vals && p.seq_lens && p.out && p.idx, SL_ERR_NULL);
+    SL_REQUIRE(p.w1_q && p.w1_k, SL_ERR_NULL);
+    if (p.lru_C > 0)
+        SL_REQUIRE(p.slot_token && p.slot_stamp && p.token_slot && p.k_res && p.v_res && p.slots_out && p.step_counter, SL_ERR_NULL);
+    return SL_OK;
+}
+
+}  // namespace
+
+extern "C" const char *sl_strerror(int status) {
+    switch (status) {
+        case SL_OK: return "ok";
+        case SL_ERR_NULL: return "a required pointer is NULL";
+        case SL_ERR_SHAPE: return "invalid size or shape";
+        case SL_ERR_UNSUPPORTED: return "shape or dtype not supported by the gfx950 kernels";
+        case SL_ERR_ALIGN: return "pointer or stride is not aligned as required";
+        case SL_ERR_WORKSPACE: return "workspace missing or too small";
+        case SL_ERR_LAUNCH: return "kernel launch failed";
+        default: return "unknown status";
+    }
+}
+
+extern "C" int sl_version(void) { return 100; }
+
+extern "C" int sl_workspace_init(void *ws, size_t ws_bytes, void *stream) {
+    if (ws_bytes == 0) return SL_OK;
+    SL_REQUIRE(ws, SL_ERR_NULL);
+    SL_REQUIRE(sl_aligned(ws, 16), SL_ERR_ALIGN);
+    const size_t n16 = ws_bytes / 16, n_tail = ws_bytes % 16;
+    size_t blocks = (n16 + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks == 0) blocks = 1;
+    fill_zero_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<uint4 *>(ws), n16, static_cast<uint8_t *>(ws) + n16 * 16, n_tail);
+    return sl_check_launch();
+}
+
+extern "C" size_t sl_decode_workspace_bytes(const sl_decode_params *p) {
+    if (!p || p->B <= 0 || p->QH <= 0 || p->KH <= 0 || p->nbits <= 0 || p->n_cap <= 0 || p->k <= 0) return 0;
+    return layout(*p).total;
+}
+
+extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
+    SL_REQUIRE(pp, SL_ERR_NULL);
+    const sl_decode_params &p = *pp;
+    int rc = validate(p);
+    if (rc != SL_OK) return rc;
+    const ws_layout L = layout(p);
+    SL_REQUIRE(p.ws && p.ws_bytes >= L.total, SL_ERR_WORKSPACE);
+    SL_REQUIRE(sl_aligned(p.ws, 256), SL_ERR_ALIGN);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    char *ws = static_cast<char *>(p.ws);
+    const int W = p.nbits / 32, G = p.QH / p.KH;
+    uint32_t *q_code = reinterpret_cast<uint32_t *>(ws + L.q_code);
+    uint32_t *hist = reinterpret_cast<uint32_t *>(ws + L.hist);
+    int16_t *score = reinterpret_cast<int16_t *>(ws + L.score);
+
+    // 1. hash q and the new key; append code, K, V
+    hash_args ha{};
+    ha.n_sides = 2;
+    ha.dtype = p.dtype; ha.n_layers = p.n_layers; ha.B = p.B; ha.d_in = p.d; ha.d_hid = p.d_hid;
+    ha.nbits = p.nbits; ha.residue = p.residue;
+    hash_side &sq = ha.side[0];
+    sq.x = p.q; sq.w1 = p.w1_q; sq.b1 = p.b1_q; sq.w2 = p.w2_q; sq.b2 = p.b2_q;
+    sq.codes = q_code; sq.code_row = nullptr; sq.H = p.QH;
+    sq.x_stride_b = static_cast<int64_t>(p.QH) * p.d;
+    sq.code_stride_b = static_cast<int64_t>(p.QH) * W; sq.code_stride_h = W; sq.code_stride_n = 0;
+    hash_side &sk = ha.side[1];
+    sk.x = p.k_new; sk.w1 = p.w1_k; sk.b1 = p.b1_k; sk.w2 = p.w2_k; sk.b2 = p.b2_k;
+    sk.codes = p.codes; sk.code_row = p.seq_lens; sk.H = p.KH;
+    sk.x_stride_b = static_cast<int64_t>(p.KH) * p.d;
+    sk.code_stride_b = p.n_cap * p.KH * W; sk.code_stride_h = W; sk.code_stride_n = static_cast<int64_t>(p.KH) * W;
+    sk.copy_src[0] = p.k_new; sk.copy_dst[0] = p.keys;
+    sk.copy_src[1] = p.v_new; sk.copy_dst[1] = p.vals;
+    sk.copy_dst_stride_b = p.n_cap * p.KH * p.d; sk.copy_dst_stride_n = static_cast<int64_t>(p.KH) * p.d;
+    rc = sl_hash_launch(ha, ws + L.hash, L.attn - L.hash, s);
+    if (rc != SL_OK) return rc;
+
+    // 2. score seq_lens[b] + 1 rows
+    hamming_args sa{};
+    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = hist; sa.seq_lens = p.seq_lens;
+    sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
+    sa.n_bins = G * p.nbits + 1; sa.len_bias = 1; sa.n = p.n_max; sa.n_cap = p.n_cap;
+    sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
+    rc = sl_hamming_launch(sa, true, s);
+    if (rc != SL_OK) return rc;
+
+    // 3. select
+    select_args ta{};
+    ta.score = score; ta.hist = hist; ta.idx = p.idx; ta.seq_lens = p.seq_lens;
+    ta.B = p.B; ta.KH = p.KH; ta.k = p.k; ta.n_bins = sa.n_bins; ta.len_bias = 1; ta.n = p.n_max;
+    ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
+    rc = sl_select_launch(ta, s);
+    if (rc != SL_OK) return rc;
+
+    // 4. optional LRU, 5. attention
+    attn_args aa{};
+    aa.q = p.q; aa.out = p.out; aa.dtype = p.dtype; aa.B = p.B; aa.QH = p.QH; aa.KH = p.KH; aa.k = p.k;
+    aa.rows = 0; aa.scale = 0.f; aa.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
+    aa.bump_lens = p.seq_lens; aa.bump_step = p.step_counter;
+    if (p.lru_C > 0) {
+        SL_REQUIRE(p.k + 1 <= p.lru_C && p.lru_C <= LRU_MAX_SLOTS, SL_ERR_UNSUPPORTED);
+        lru_args la{};
+        la.idx = p.idx; la.new_token = p.seq_lens; la.slot_token = p.slot_token; la.slot_stamp = p.slot_stamp;
+        la.token_slot = p.token_slot; la.keys = p.keys; la.vals = p.vals; la.k_res = p.k_res; la.v_res = p.v_res;
+        la.slots_out = p.slots_out; la.stats = p.lru_stats; la.stamp_dev = p.step_counter; la.stamp = 1;
+        la.dtype = p.dtype; la.B = p.B; la.KH = p.KH; la.d = p.d; la.k = p.k; la.C = p.lru_C;
+        la.map_cap = p.lru_map_cap; la.kv_stride_b = p.n_cap * p.KH * p.d;
+        rc = sl_lru_launch(la, s);
+        if (rc != SL_OK) return rc;
+        aa.keys = p.k_res; aa.vals = p.v_res; aa.idx = p.slots_out;
+        aa.kv_stride_b = static_cast<int64_t>(p.KH) * p.lru_C * p.d;
+        aa.kv_stride_h = static_cast<int64_t>(p.lru_C) * p.d;
+        aa.kv_stride_n = p.d;
+    } else {
+        aa.keys = p.keys; aa.vals = p.vals; aa.idx = p.idx;
+        aa.kv_stride_b = p.n_cap * p.KH * p.d; aa.kv_stride_h = p.d;
+        aa.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
+    }
+    return sl_attn_launch(aa, ws + L.attn, L.total - L.attn, s);
+}
