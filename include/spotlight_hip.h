@@ -73,7 +73,8 @@ int sl_pack_sign_u8(const void *x, int dtype, uint8_t *out, int64_t n_bytes, voi
  * code_row[b] (may be NULL, then 0) is added to the code row index, in units
  * of code_stride_n, so that a key code lands in cache row seq_len[b].
  * ws: sl_hash_workspace_bytes(B, H, d_hid, nbits) bytes, zeroed once with
- * sl_workspace_init(); the kernel leaves it zeroed again. */
+ * sl_workspace_init(); its first 16 KiB (arrival tickets, H <= 4096) are left
+ * zeroed, so one workspace can serve calls of any shape it is big enough for. */
 size_t sl_hash_workspace_bytes(int B, int H, int d_hid, int nbits);
 int sl_hash_mlp_pack(const void *x, const void *w1, const void *b1, const void *w2,
                      const void *b2, uint32_t *codes, int dtype, int n_layers, int B,
@@ -175,7 +176,10 @@ int sl_lru_update(const int32_t *idx, const int32_t *new_token, int32_t *slot_to
  *   idx  [B, KH, k] int32 row numbers (negative entries are skipped)
  *   out  [B, QH, d] dtype contiguous; kv head of q head qh is qh / G.
  * d must be 128.  fp32 softmax and accumulation; scale <= 0 means 1/sqrt(d).
- * ws: sl_attn_workspace_bytes(B, QH, KH, d, k), zeroed once; left zeroed. */
+ * ws: sl_attn_workspace_bytes(B, QH, KH, d, k) bytes, zeroed once with
+ * sl_workspace_init(); its first 64 KiB (arrival tickets, B*KH <= 16384) are
+ * left zeroed, so one workspace can serve calls of any shape it is big
+ * enough for. */
 size_t sl_attn_workspace_bytes(int B, int QH, int KH, int d, int k);
 int sl_sparse_gqa_attn(const void *q, const void *keys, const void *vals, const int32_t *idx,
                        void *out, int dtype, int B, int QH, int KH, int d, int k,

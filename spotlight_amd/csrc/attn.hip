@@ -20,6 +20,10 @@ namespace {
 constexpr int AT_THREADS = 256;
 constexpr int AT_D = 128;
 constexpr int AT_PART = AT_D + 2;  // acc[128], m, l
+// The arrival tickets sit in a fixed-size head of the workspace so that the
+// partials of a call with other shapes can never land on them: the tickets are
+// the only part that has to stay zero between calls.
+constexpr size_t AT_COUNTER_BYTES = 64 * 1024;
 
 template <typename T, int G, int STEPS>
 __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
@@ -240,15 +244,15 @@ size_t sl_attn_ws_bytes(int B, int QH, int KH, int k) {
     const size_t bh = static_cast<size_t>(B) * KH;
     const size_t S = (static_cast<size_t>(k) + 15) / 16;
     const size_t G = static_cast<size_t>(QH / KH);
-    return sl_align_up(bh * sizeof(uint32_t), 256) + sl_align_up(bh * S * G * AT_PART * sizeof(float), 256);
+    return AT_COUNTER_BYTES + sl_align_up(bh * S * G * AT_PART * sizeof(float), 256);
 }
 
 int sl_attn_launch(attn_args a, void *ws, size_t ws_bytes, hipStream_t s) {
     SL_REQUIRE(ws && ws_bytes >= sl_attn_ws_bytes(a.B, a.QH, a.KH, a.k), SL_ERR_WORKSPACE);
     SL_REQUIRE(sl_aligned(ws, 16), SL_ERR_ALIGN);
     a.counter = static_cast<uint32_t *>(ws);
-    a.part = reinterpret_cast<float *>(static_cast<char *>(ws) +
-                                       sl_align_up(static_cast<size_t>(a.B) * a.KH * sizeof(uint32_t), 256));
+    SL_REQUIRE(static_cast<size_t>(a.B) * a.KH * sizeof(uint32_t) <= AT_COUNTER_BYTES, SL_ERR_UNSUPPORTED);
+    a.part = reinterpret_cast<float *>(static_cast<char *>(ws) + AT_COUNTER_BYTES);
     if (a.rows == 0) a.rows = pick_rows(a.B, a.KH, a.k);
     if (a.scale <= 0.f) a.scale = 0.08838834764831845f;  // 1/sqrt(128)
     switch (a.dtype) {

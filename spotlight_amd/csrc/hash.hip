@@ -25,6 +25,9 @@ constexpr int HK_SLICE = 64;   // hidden units per workgroup
 constexpr int HK_BT = 4;       // batch rows per pass
 constexpr int HK_DIN = 128;
 constexpr int HK_NBITS = 128;
+// Arrival tickets live in a fixed-size head of the workspace: they are the only
+// part that must stay zero between calls, whatever the shapes of those calls.
+constexpr size_t HK_COUNTER_BYTES = 16 * 1024;
 
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
@@ -211,7 +214,7 @@ int launch(const hash_args &a, int Htot, hipStream_t s) {
 size_t sl_hash_ws_bytes(int B, int Htot, int d_hid, int nbits) {
     if (B <= 0 || Htot <= 0 || d_hid <= 0 || nbits <= 0) return 0;
     const size_t slices = static_cast<size_t>(d_hid + HK_SLICE - 1) / HK_SLICE;
-    return sl_align_up(sizeof(uint32_t) * Htot, 256) +
+    return HK_COUNTER_BYTES +
            sl_align_up(sizeof(float) * static_cast<size_t>(B) * Htot * slices * nbits, 256) +
            sl_align_up(sizeof(float) * static_cast<size_t>(B) * Htot * d_hid, 256);
 }
@@ -240,12 +243,12 @@ int sl_hash_launch(hash_args a, void *ws, size_t ws_bytes, hipStream_t s) {
             }
         Htot += sd.H;
     }
-    SL_REQUIRE(Htot <= 65535, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(Htot * sizeof(uint32_t) <= HK_COUNTER_BYTES, SL_ERR_UNSUPPORTED);
     SL_REQUIRE(ws && ws_bytes >= sl_hash_ws_bytes(a.B, Htot, a.d_hid, a.nbits), SL_ERR_WORKSPACE);
     SL_REQUIRE(sl_aligned(ws, 16), SL_ERR_ALIGN);
     char *p = static_cast<char *>(ws);
     a.counter = reinterpret_cast<uint32_t *>(p);
-    p += sl_align_up(sizeof(uint32_t) * Htot, 256);
+    p += HK_COUNTER_BYTES;
     a.part = reinterpret_cast<float *>(p);
     const size_t slices = static_cast<size_t>(a.d_hid) / HK_SLICE;
     p += sl_align_up(sizeof(float) * static_cast<size_t>(a.B) * Htot * slices * a.nbits, 256);

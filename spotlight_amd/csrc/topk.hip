@@ -24,14 +24,17 @@ constexpr int TK_RUN = 8;
 constexpr int TK_PASS_TOKENS = TK_THREADS * TK_RUN;  // tokens per chunk (8192)
 
 // ---- histogram of externally produced scores -------------------------------
-// One workgroup per (token block, b); LDS histogram per head, then flush.
+// One workgroup per (token block, b, group of heads whose bins fit 64 KiB of
+// LDS); LDS histogram per head, then flush.
 constexpr int SH_THREADS = 256;
 constexpr int SH_TOKENS = 512;  // tokens per workgroup
 
-__global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a) {
+__global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, int heads_per_group) {
     extern __shared__ uint32_t hist[];
     const int b = blockIdx.y;
-    const int KH = a.KH, NB = a.n_bins;
+    const int NB = a.n_bins;
+    const int h0 = blockIdx.z * heads_per_group;
+    const int KHg = a.KH - h0 < heads_per_group ? a.KH - h0 : heads_per_group;  // heads of this group
     int64_t n_b = a.n;
     if (a.seq_lens) {
         const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
@@ -39,22 +42,22 @@ __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a) {
     }
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * SH_TOKENS;
     if (t0 >= n_b) return;
-    for (int e = threadIdx.x; e < KH * NB; e += SH_THREADS) hist[e] = 0;
+    for (int e = threadIdx.x; e < KHg * NB; e += SH_THREADS) hist[e] = 0;
     __syncthreads();
     const int64_t rem = n_b - t0;
     const int nt = rem < SH_TOKENS ? static_cast<int>(rem) : SH_TOKENS;
     const int16_t *sb = a.score + static_cast<int64_t>(b) * a.stride_b;
     const bool token_major = a.stride_h <= a.stride_n;
-    for (int e = threadIdx.x; e < nt * KH; e += SH_THREADS) {
-        const int tl = token_major ? e / KH : e % nt;
-        const int h = token_major ? e % KH : e / nt;
-        int s = sb[(t0 + tl) * a.stride_n + h * a.stride_h];
+    for (int e = threadIdx.x; e < nt * KHg; e += SH_THREADS) {
+        const int tl = token_major ? e / KHg : e % nt;
+        const int h = token_major ? e % KHg : e / nt;
+        int s = sb[(t0 + tl) * a.stride_n + (h0 + h) * a.stride_h];
         s = s < 0 ? 0 : (s >= NB ? NB - 1 : s);
         atomicAdd(&hist[h * NB + s], 1u);
     }
     __syncthreads();
-    uint32_t *gh = a.hist + static_cast<int64_t>(b) * KH * NB;
-    for (int i = threadIdx.x; i < KH * NB; i += SH_THREADS) {
+    uint32_t *gh = a.hist + (static_cast<int64_t>(b) * a.KH + h0) * NB;
+    for (int i = threadIdx.x; i < KHg * NB; i += SH_THREADS) {
         const uint32_t c = hist[i];
         if (c) atomicAdd(&gh[i], c);
     }
@@ -215,16 +218,19 @@ extern "C" int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t st
     SL_REQUIRE(n <= 0x7fffffffLL && B <= 65535, SL_ERR_UNSUPPORTED);
     SL_REQUIRE(ws && ws_bytes >= sl_topk_workspace_bytes(B, KH, max_score), SL_ERR_WORKSPACE);
     SL_REQUIRE(sl_aligned(ws, 4), SL_ERR_ALIGN);
-    const size_t lds = sizeof(uint32_t) * static_cast<size_t>(KH) * (max_score + 1);
-    SL_REQUIRE(lds <= 64 * 1024, SL_ERR_UNSUPPORTED);
+    const int n_bins = max_score + 1;
+    int heads_per_group = 16384 / n_bins;  // 64 KiB of LDS bins per workgroup
+    if (heads_per_group > KH) heads_per_group = KH;
+    const int groups = (KH + heads_per_group - 1) / heads_per_group;
+    const size_t lds = sizeof(uint32_t) * static_cast<size_t>(heads_per_group) * n_bins;
     select_args a{};
     a.score = score; a.hist = static_cast<uint32_t *>(ws); a.idx = idx; a.seq_lens = seq_lens;
     a.B = B; a.KH = KH; a.k = k; a.n_bins = max_score + 1; a.len_bias = 0; a.n = n;
     a.stride_b = stride_b; a.stride_n = stride_n; a.stride_h = stride_h;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n > 0) {
-        const dim3 grid(static_cast<unsigned>((n + SH_TOKENS - 1) / SH_TOKENS), B);
-        score_hist_kernel<<<grid, dim3(SH_THREADS), lds, s>>>(a);
+        const dim3 grid(static_cast<unsigned>((n + SH_TOKENS - 1) / SH_TOKENS), B, groups);
+        score_hist_kernel<<<grid, dim3(SH_THREADS), lds, s>>>(a, heads_per_group);
         const int rc = sl_check_launch();
         if (rc != SL_OK) return rc;
     }

@@ -1,0 +1,217 @@
+"""Per-layer decode state driving the fused HIP decode step.
+
+One ``LayerDecodeState`` owns what one attention layer needs between decode
+steps: packed key codes, K and V (token-major ``[B, n_cap, KH, .]`` like the
+reference's ``KVHash`` / ``KVCache`` buffers, spotlight/modifiers/gpu_cache.py:
+27-36,77-95), the per-sequence lengths on the device, the hash weights of both
+sides and the scratch workspace.  ``step`` is the kernel-path composition of
+the reference's decode branch (spotlight/modifiers/spotlight_generation.py:
+143-215): hash -> pack -> score -> top-k -> (LRU) -> sparse attention.
+
+All lengths live on the device, so a captured HIP graph of ``step`` can be
+replayed while the cache grows (``capture`` / ``replay``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+from . import kernel as K
+
+_L = _lib.load()
+
+
+@dataclass
+class HashWeights:
+    """Per-head hash weights of one side (query or key).
+
+    Two layers: ``w1 [H,d,d_hid]``, ``b1 [H,d_hid]``, ``w2 [H,d_hid,nbits]``,
+    ``b2 [H,nbits]`` -- the ``proj`` / ``bias`` of MLPLayer squeezed of their
+    unit dimensions (spotlight_generation.py:232-234).  One layer (linear
+    hashing, linearhashing_generation.py:227): ``w1 [H,d,nbits]`` only."""
+    w1: torch.Tensor
+    b1: Optional[torch.Tensor] = None
+    w2: Optional[torch.Tensor] = None
+    b2: Optional[torch.Tensor] = None
+    residue: bool = False
+
+    @property
+    def n_layers(self) -> int:
+        return 2 if self.w2 is not None else 1
+
+    @property
+    def d_hid(self) -> int:
+        return self.w1.shape[2]
+
+    @property
+    def nbits(self) -> int:
+        return self.w2.shape[2] if self.w2 is not None else self.w1.shape[2]
+
+    @staticmethod
+    def random_mlp(H, dims, dtype, device, generator=None, scale=0.001, residue=False):
+        """The reference's init: proj ~ N(0,1)*0.001, bias = 0 (spotlight_generation.py:232-234)."""
+        assert len(dims) == 3
+        w = [(torch.randn(H, dims[i], dims[i + 1], generator=generator) * scale).to(dtype).to(device)
+             for i in range(2)]
+        b = [torch.zeros(H, dims[i + 1], dtype=dtype, device=device) for i in range(2)]
+        return HashWeights(w[0], b[0], w[1], b[1], residue)
+
+    @staticmethod
+    def random_linear(H, d, nbits, dtype, device, generator=None):
+        """Gaussian projection, not orthogonalised (linearhashing_generation.py:227)."""
+        return HashWeights(torch.randn(H, d, nbits, generator=generator).to(dtype).to(device))
+
+    def hash_rows(self, x: torch.Tensor) -> torch.Tensor:
+        """Codes of many rows per head (prefill): x [B,n,H,d] -> uint32 [B,n,H,nbits/32].
+
+        Library GEMMs for the projections (this is GEMM-shaped work), then the
+        HIP pack kernel; rounding follows the reference's torch expression."""
+        B, n, H, d = x.shape
+        h = x.permute(2, 0, 1, 3).reshape(H, B * n, d)
+        y = torch.bmm(h, self.w1)
+        if self.b1 is not None:
+            y = y + self.b1[:, None, :]
+        if self.w2 is not None:
+            y = torch.nn.functional.silu(y)
+            if self.residue:
+                y = y + h
+            z = torch.bmm(y, self.w2)
+            if self.b2 is not None:
+                z = z + self.b2[:, None, :]
+            if self.residue:
+                z = z + y
+        else:
+            z = y + h if self.residue else y
+        z = z.reshape(H, B, n, -1).permute(1, 2, 0, 3).contiguous()
+        return K.pack_cuda_func(z)
+
+
+class LayerDecodeState:
+    def __init__(self, batch_size: int, num_heads: int, num_kv_heads: int, head_dim: int, n_cap: int, k: int,
+                 hash_q: HashWeights, hash_k: HashWeights, dtype=torch.bfloat16, device="cuda",
+                 head_map: str = "blocked", lru_slots: int = 0):
+        assert head_dim == 128, "the attention kernel covers head_dim 128"
+        assert n_cap % 8 == 0, "n_cap must be a multiple of 8"
+        assert hash_q.nbits == hash_k.nbits and hash_q.n_layers == hash_k.n_layers
+        assert hash_q.d_hid == hash_k.d_hid and hash_q.residue == hash_k.residue
+        self.B, self.QH, self.KH, self.d = batch_size, num_heads, num_kv_heads, head_dim
+        self.n_cap, self.k, self.dtype, self.device = n_cap, k, dtype, torch.device(device)
+        self.nbits = hash_q.nbits
+        self.W = self.nbits // 32
+        self.hash_q, self.hash_k = hash_q, hash_k
+        self.head_map = head_map
+        dev = self.device
+        B, QH, KH, d, W = self.B, self.QH, self.KH, self.d, self.W
+        self.codes = torch.zeros((B, n_cap, KH, W), dtype=torch.uint32, device=dev)
+        self.keys = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=dev)
+        self.vals = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=dev)
+        self.seq_lens = torch.zeros((B,), dtype=torch.int32, device=dev)
+        self.step_counter = torch.zeros((1,), dtype=torch.int32, device=dev)
+        self.q_in = torch.zeros((B, QH, d), dtype=dtype, device=dev)
+        self.k_in = torch.zeros((B, KH, d), dtype=dtype, device=dev)
+        self.v_in = torch.zeros((B, KH, d), dtype=dtype, device=dev)
+        self.out = torch.zeros((B, QH, d), dtype=dtype, device=dev)
+        self.idx = torch.full((B, KH, k), -1, dtype=torch.int32, device=dev)
+        self.host_len = 0  # upper bound of seq_lens, tracked on the host for grid sizing
+        self.lru_slots = lru_slots
+        if lru_slots:
+            assert k + 1 <= lru_slots <= 4096
+            self.slot_token = torch.full((B, KH, lru_slots), -1, dtype=torch.int32, device=dev)
+            self.slot_stamp = torch.zeros((B, KH, lru_slots), dtype=torch.int32, device=dev)
+            self.token_slot = torch.full((B, KH, n_cap), -1, dtype=torch.int32, device=dev)
+            self.k_res = torch.zeros((B, KH, lru_slots, d), dtype=dtype, device=dev)
+            self.v_res = torch.zeros((B, KH, lru_slots, d), dtype=dtype, device=dev)
+            self.slots_out = torch.full((B, KH, k), -1, dtype=torch.int32, device=dev)
+            self.lru_stats = torch.zeros((B, KH, 2), dtype=torch.int32, device=dev)
+        self.params = self._make_params()
+        nbytes = _L.sl_decode_workspace_bytes(C.byref(self.params))
+        assert nbytes > 0
+        self.ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            _lib.check(_L.sl_workspace_init(self.ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream),
+                       "sl_workspace_init")
+        self.params.ws = self.ws.data_ptr()
+        self.params.ws_bytes = nbytes
+        self._graph = None
+
+    def _make_params(self) -> _lib.DecodeParams:
+        p = _lib.DecodeParams()
+        p.dtype = K._DTYPES[self.dtype]
+        p.B, p.QH, p.KH, p.d = self.B, self.QH, self.KH, self.d
+        p.nbits, p.k = self.nbits, self.k
+        p.head_map = K._HEAD_MAPS[self.head_map]
+        p.n_cap, p.n_max = self.n_cap, 1
+        p.q, p.k_new, p.v_new = self.q_in.data_ptr(), self.k_in.data_ptr(), self.v_in.data_ptr()
+        hq, hk = self.hash_q, self.hash_k
+        p.n_layers, p.d_hid, p.residue = hq.n_layers, hq.d_hid, int(hq.residue)
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        p.w1_q, p.b1_q, p.w2_q, p.b2_q = ptr(hq.w1), ptr(hq.b1), ptr(hq.w2), ptr(hq.b2)
+        p.w1_k, p.b1_k, p.w2_k, p.b2_k = ptr(hk.w1), ptr(hk.b1), ptr(hk.w2), ptr(hk.b2)
+        p.codes, p.keys, p.vals = self.codes.data_ptr(), self.keys.data_ptr(), self.vals.data_ptr()
+        p.seq_lens, p.out, p.idx = self.seq_lens.data_ptr(), self.out.data_ptr(), self.idx.data_ptr()
+        p.step_counter = self.step_counter.data_ptr()
+        p.lru_C = self.lru_slots
+        if self.lru_slots:
+            p.lru_map_cap = self.n_cap
+            p.slot_token, p.slot_stamp = self.slot_token.data_ptr(), self.slot_stamp.data_ptr()
+            p.token_slot = self.token_slot.data_ptr()
+            p.k_res, p.v_res = self.k_res.data_ptr(), self.v_res.data_ptr()
+            p.slots_out, p.lru_stats = self.slots_out.data_ptr(), self.lru_stats.data_ptr()
+        return p
+
+    # -- prefill ---------------------------------------------------------------
+    def prefill(self, keys: torch.Tensor, vals: torch.Tensor, codes: Optional[torch.Tensor] = None) -> None:
+        """Store n0 post-RoPE rows per sequence: keys/vals [B,n0,KH,d]; codes
+        [B,n0,KH,W] are hashed from the keys when not given."""
+        n0 = keys.shape[1]
+        assert self.host_len == 0 and n0 < self.n_cap
+        if codes is None:
+            codes = self.hash_k.hash_rows(keys)
+        K.cache_append(self.keys, keys.contiguous())
+        K.cache_append(self.vals, vals.contiguous())
+        K.cache_append(self.codes, codes.contiguous())
+        self.seq_lens.fill_(n0)
+        self.host_len = n0
+
+    # -- decode ------------------------------------------------------------------
+    def _launch(self, n_max: int) -> None:
+        if n_max > self.n_cap:
+            raise RuntimeError(f"cache capacity {self.n_cap} exceeded")
+        self.params.n_max = n_max
+        _lib.check(_L.sl_decode_step(C.byref(self.params), torch.cuda.current_stream().cuda_stream),
+                   "sl_decode_step")
+
+    def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor) -> torch.Tensor:
+        """One decode step: q [B,QH,d], k_new/v_new [B,KH,d] (post-RoPE).
+        Returns the attention output [B,QH,d] (a buffer reused by the next step)."""
+        with torch.cuda.device(self.device):
+            self.q_in.copy_(q)
+            self.k_in.copy_(k_new)
+            self.v_in.copy_(v_new)
+            self._launch(self.host_len + 1)
+        self.host_len += 1
+        return self.out
+
+    def capture(self, steps_ahead: int) -> None:
+        """Capture one step as a HIP graph valid for the next ``steps_ahead``
+        replays (grids are sized for the longest length in that window).
+        Inputs are read from ``q_in`` / ``k_in`` / ``v_in``."""
+        n_max = min(self.host_len + steps_ahead, self.n_cap)
+        self._graph_budget = n_max - self.host_len
+        with torch.cuda.device(self.device):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._launch(n_max)
+        self._graph = g
+
+    def replay(self) -> torch.Tensor:
+        if self._graph is None or self._graph_budget <= 0:
+            raise RuntimeError("capture() a graph that covers this step first")
+        self._graph.replay()
+        self._graph_budget -= 1
+        self.host_len += 1
+        return self.out

@@ -1,0 +1,273 @@
+"""Parity of the fused decode step (hash -> score -> top-k -> (LRU) -> attention)
+and of the LRU resident table against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import spotlight_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+@pytest.fixture(scope="module")
+def env():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from spotlight_amd import decode, kernel
+    return decode, kernel
+
+
+def _gen(seed):
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def _make_state(decode, g, B, QH, KH, n0, n_cap, k, dtype, kind="mlp", lru=0, scale=0.05, head_map="blocked"):
+    if kind == "mlp":
+        hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, DEV, g, scale=scale)
+        hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, DEV, g, scale=scale)
+    else:
+        hq = decode.HashWeights.random_linear(QH, 128, 128, dtype, DEV, g)
+        hk = hq if KH == QH else decode.HashWeights.random_linear(KH, 128, 128, dtype, DEV, g)
+    st = decode.LayerDecodeState(B, QH, KH, 128, n_cap, k, hq, hk, dtype=dtype, device=DEV,
+                                 head_map=head_map, lru_slots=lru)
+    keys = torch.randn(B, n0, KH, 128, generator=g).to(dtype)
+    vals = torch.randn(B, n0, KH, 128, generator=g).to(dtype)
+    st.prefill(keys.to(DEV), vals.to(DEV))
+    return st
+
+
+def _check_step(kernel, st, q, k_new, v_new, out, n_before, dtype):
+    """Everything the step produced, checked against the oracle on the codes the GPU holds."""
+    B, QH, KH = st.B, st.QH, st.KH
+    n = n_before + 1
+    hq = st.hash_q
+    q_code = kernel.hash_mlp_pack(q.to(DEV), hq.w1, hq.b1, hq.w2, hq.b2, hq.residue).cpu().numpy()[:, None]
+    codes = st.codes[:, :n].cpu().numpy()
+    keys = st.keys[:, :n].float().cpu().numpy()
+    vals = st.vals[:, :n].float().cpu().numpy()
+    # appended row
+    np.testing.assert_array_equal(keys[:, n - 1], k_new.float().numpy())
+    np.testing.assert_array_equal(vals[:, n - 1], v_new.float().numpy())
+    hk = st.hash_k
+    k_code = kernel.hash_mlp_pack(k_new.to(DEV), hk.w1, hk.b1, hk.w2, hk.b2, hk.residue).cpu().numpy()
+    np.testing.assert_array_equal(codes[:, n - 1], k_code)
+    assert st.seq_lens.cpu().tolist() == [n] * B
+    # selection: bit exact
+    score = orc.hamming_score_u32(q_code, codes, st.head_map)
+    want_idx = orc.topk_stable(score, st.k)
+    got_idx = st.idx.cpu().numpy()
+    kk = want_idx.shape[2]
+    np.testing.assert_array_equal(got_idx[:, :, :kk], want_idx)
+    assert (got_idx[:, :, kk:] == -1).all()
+    # attention
+    want = orc.sparse_attention(q.float().numpy(), keys, vals, want_idx)
+    err = np.abs(out.float().cpu().numpy() - want).max()
+    assert err <= TOL[dtype], err
+
+
+DECODE_CASES = [
+    # B, QH, KH, n0, k, dtype, kind
+    (1, 32, 8, 1000, 20, torch.bfloat16, "mlp"),
+    (1, 32, 8, 2047, 41, torch.float32, "mlp"),
+    (2, 40, 8, 777, 16, torch.bfloat16, "mlp"),
+    (1, 32, 32, 512, 52, torch.float32, "linear"),     # Llama-2 shape, training-free hash (config 1 style)
+    (3, 28, 4, 300, 30, torch.float16, "mlp"),
+    (1, 8, 8, 5, 20, torch.float32, "mlp"),            # fewer tokens than k
+]
+
+
+@pytest.mark.parametrize("B,QH,KH,n0,k,dtype,kind", DECODE_CASES)
+def test_decode_step_matches_oracle(env, B, QH, KH, n0, k, dtype, kind):
+    decode, kernel = env
+    g = _gen(n0 + k)
+    st = _make_state(decode, g, B, QH, KH, n0, 2048 + 64, k, dtype, kind)
+    for step in range(3):
+        q = torch.randn(B, QH, 128, generator=g).to(dtype)
+        k_new = torch.randn(B, KH, 128, generator=g).to(dtype)
+        v_new = torch.randn(B, KH, 128, generator=g).to(dtype)
+        out = st.step(q.to(DEV), k_new.to(DEV), v_new.to(DEV))
+        _check_step(kernel, st, q, k_new, v_new, out, n0 + step, dtype)
+
+
+def test_decode_step_interleaved_head_map(env):
+    decode, kernel = env
+    g = _gen(77)
+    st = _make_state(decode, g, 1, 28, 4, 400, 512, 25, torch.bfloat16, head_map="interleaved")
+    q = torch.randn(1, 28, 128, generator=g).to(torch.bfloat16)
+    kn = torch.randn(1, 4, 128, generator=g).to(torch.bfloat16)
+    vn = torch.randn(1, 4, 128, generator=g).to(torch.bfloat16)
+    out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV))
+    _check_step(kernel, st, q, kn, vn, out, 400, torch.bfloat16)
+
+
+def test_decode_ragged_batch(env):
+    """Sequences of different lengths in one batch (lengths live on the device)."""
+    decode, kernel = env
+    g = _gen(78)
+    B, QH, KH, k = 3, 32, 8, 24
+    st = _make_state(decode, g, B, QH, KH, 600, 1024, k, torch.float32)
+    lens = [600, 77, 333]
+    st.seq_lens.copy_(torch.tensor(lens, dtype=torch.int32))
+    q = torch.randn(B, QH, 128, generator=g)
+    kn = torch.randn(B, KH, 128, generator=g)
+    vn = torch.randn(B, KH, 128, generator=g)
+    out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).cpu().numpy()
+    hq = st.hash_q
+    q_code = kernel.hash_mlp_pack(q.to(DEV), hq.w1, hq.b1, hq.w2, hq.b2).cpu().numpy()[:, None]
+    assert st.seq_lens.cpu().tolist() == [l + 1 for l in lens]
+    for b, l in enumerate(lens):
+        n = l + 1
+        codes = st.codes[b:b + 1, :n].cpu().numpy()
+        score = orc.hamming_score_u32(q_code[b:b + 1], codes, "blocked")
+        want_idx = orc.topk_stable(score, k)
+        np.testing.assert_array_equal(st.idx[b:b + 1].cpu().numpy(), want_idx)
+        want = orc.sparse_attention(q[b:b + 1].numpy(), st.keys[b:b + 1, :n].cpu().numpy(),
+                                    st.vals[b:b + 1, :n].cpu().numpy(), want_idx)
+        assert np.abs(out[b:b + 1] - want).max() <= 1e-5
+
+
+def test_decode_graph_replay_equals_eager(env):
+    """A captured step replayed while the cache grows gives what eager steps give."""
+    decode, kernel = env
+    dtype = torch.bfloat16
+    states = [_make_state(decode, _gen(90), 2, 32, 8, 500, 640, 30, dtype) for _ in range(2)]
+    eager, graphed = states
+    graphed.capture(steps_ahead=8)
+    g = _gen(91)
+    for step in range(6):
+        q = torch.randn(2, 32, 128, generator=g).to(dtype).to(DEV)
+        kn = torch.randn(2, 8, 128, generator=g).to(dtype).to(DEV)
+        vn = torch.randn(2, 8, 128, generator=g).to(dtype).to(DEV)
+        a = eager.step(q, kn, vn).clone()
+        graphed.q_in.copy_(q); graphed.k_in.copy_(kn); graphed.v_in.copy_(vn)
+        b = graphed.replay().clone()
+        torch.cuda.synchronize()
+        assert torch.equal(eager.idx, graphed.idx), step
+        assert torch.equal(a, b), step
+        assert torch.equal(eager.seq_lens, graphed.seq_lens)
+    with pytest.raises(RuntimeError):
+        for _ in range(5):
+            graphed.replay()
+
+
+def test_decode_is_deterministic(env):
+    decode, kernel = env
+    outs = []
+    for _ in range(2):
+        g = _gen(95)
+        st = _make_state(decode, g, 1, 32, 8, 3000, 3072, 60, torch.bfloat16)
+        q = torch.randn(1, 32, 128, generator=g).to(torch.bfloat16)
+        kn = torch.randn(1, 8, 128, generator=g).to(torch.bfloat16)
+        vn = torch.randn(1, 8, 128, generator=g).to(torch.bfloat16)
+        outs.append((st.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).clone(), st.idx.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+# ---- LRU ---------------------------------------------------------------------------------
+
+def _lru_call(kernel, lib, L, idx, new_tok, st, ss, ts, keys, vals, kres, vres, stamp):
+    B, KH, k = idx.shape
+    C = st.shape[2]
+    slots = torch.full((B, KH, k), -7, dtype=torch.int32, device=DEV)
+    stats = torch.zeros((B, KH, 2), dtype=torch.int32, device=DEV)
+    rc = L.sl_lru_update(idx.data_ptr(), new_tok.data_ptr(), st.data_ptr(), ss.data_ptr(), ts.data_ptr(),
+                         keys.data_ptr(), vals.data_ptr(), kres.data_ptr(), vres.data_ptr(), slots.data_ptr(),
+                         stats.data_ptr(), kernel._DTYPES[keys.dtype], B, KH, keys.shape[3], k, C, ts.shape[2],
+                         keys.stride(0), stamp, None, torch.cuda.current_stream().cuda_stream)
+    lib.check(rc, "sl_lru_update")
+    return slots, stats
+
+
+@pytest.mark.parametrize("C,k,n0,steps", [(8, 3, 12, 40), (64, 20, 100, 30), (1024, 328, 2000, 6), (4096, 1000, 5000, 3)])
+def test_lru_matches_bruteforce_model(env, C, k, n0, steps):
+    decode, kernel = env
+    from spotlight_amd import _lib as lib
+    L = lib.load()
+    r = np.random.default_rng(C + k)
+    B, KH, d = 2, 3, 128
+    cap = n0 + steps + 1
+    keys = torch.randn(B, cap, KH, d, generator=_gen(1)).to(torch.bfloat16).to(DEV)
+    vals = torch.randn(B, cap, KH, d, generator=_gen(2)).to(torch.bfloat16).to(DEV)
+    st = torch.full((B, KH, C), -1, dtype=torch.int32, device=DEV)
+    ss = torch.zeros((B, KH, C), dtype=torch.int32, device=DEV)
+    ts = torch.full((B, KH, cap), -1, dtype=torch.int32, device=DEV)
+    kres = torch.zeros((B, KH, C, d), dtype=torch.bfloat16, device=DEV)
+    vres = torch.zeros_like(kres)
+    models = [[orc.LruModel(C) for _ in range(KH)] for _ in range(B)]
+    n = n0
+    for t in range(1, steps + 1):
+        idx = np.zeros((B, KH, k), dtype=np.int32)
+        for b in range(B):
+            for h in range(KH):
+                sel = r.choice(n, size=k, replace=False)
+                res = [x for x in models[b][h].token if x >= 0]
+                if res and t % 2 == 0:      # re-use resident tokens so that hits occur
+                    take = min(len(res), k // 2)
+                    sel = np.unique(np.concatenate([r.choice(res, size=take, replace=False), sel]))[:k]
+                    while len(sel) < k:
+                        sel = np.unique(np.concatenate([sel, r.choice(n, size=k)]))[:k]
+                idx[b, h] = np.sort(sel)
+        new_tok = torch.full((B,), n, dtype=torch.int32, device=DEV)
+        slots, stats = _lru_call(kernel, lib, L, torch.from_numpy(idx).to(DEV), new_tok, st, ss, ts, keys, vals,
+                                 kres, vres, t)
+        slots = slots.cpu().numpy()
+        st_h, ss_h, ts_h = st.cpu().numpy(), ss.cpu().numpy(), ts.cpu().numpy()
+        stats = stats.cpu().numpy()
+        for b in range(B):
+            for h in range(KH):
+                m = models[b][h]
+                h0, m0 = m.hits, m.misses
+                want_slots = m.step(t, idx[b, h], n)
+                assert st_h[b, h].tolist() == m.token, (t, b, h)
+                assert ss_h[b, h].tolist() == m.stamp, (t, b, h)
+                assert slots[b, h].tolist() == want_slots
+                assert stats[b, h].tolist() == [m.hits - h0, m.misses - m0]
+                inv = np.full(cap, -1, dtype=np.int32)
+                for s, tok in enumerate(m.token):
+                    if tok >= 0:
+                        inv[tok] = s
+                np.testing.assert_array_equal(ts_h[b, h], inv)
+        # resident rows hold the rows of the tokens they claim to hold
+        tok = st.long().clamp(min=0)
+        want_k = torch.gather(keys.permute(0, 2, 1, 3), 2, tok.unsqueeze(-1).expand(-1, -1, -1, d))
+        want_v = torch.gather(vals.permute(0, 2, 1, 3), 2, tok.unsqueeze(-1).expand(-1, -1, -1, d))
+        live = (st >= 0).unsqueeze(-1)
+        assert torch.equal(torch.where(live, kres, 0), torch.where(live, want_k, 0))
+        assert torch.equal(torch.where(live, vres, 0), torch.where(live, want_v, 0))
+        n += 1
+
+
+def test_decode_with_lru_gives_identical_attention(env):
+    """The LRU layer changes where rows are read from, never the result."""
+    decode, kernel = env
+    dtype = torch.bfloat16
+    plain = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype)
+    lru = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype, lru=64)
+    models = [[orc.LruModel(64) for _ in range(8)] for _ in range(2)]
+    g = _gen(61)
+    for step in range(1, 9):
+        q = torch.randn(2, 32, 128, generator=g).to(dtype).to(DEV)
+        if step % 2 == 0:
+            q = prev_q          # repeat the query: the second time most selected rows are hits
+        prev_q = q
+        kn = torch.randn(2, 8, 128, generator=g).to(dtype).to(DEV)
+        vn = torch.randn(2, 8, 128, generator=g).to(dtype).to(DEV)
+        a = plain.step(q, kn, vn).clone()
+        b = lru.step(q, kn, vn).clone()
+        assert torch.equal(plain.idx, lru.idx)
+        assert torch.equal(a, b), step
+        idx = lru.idx.cpu().numpy()
+        toks, stamps = lru.slot_token.cpu().numpy(), lru.slot_stamp.cpu().numpy()
+        for bb in range(2):
+            for h in range(8):
+                m = models[bb][h]
+                m.step(step, idx[bb, h], 900 + step - 1)
+                assert toks[bb, h].tolist() == m.token and stamps[bb, h].tolist() == m.stamp
+    stats = lru.lru_stats.cpu().numpy()
+    assert stats[..., 0].sum() > 0 and stats[..., 1].sum() > 0
+    assert stats.sum() == sum(m.hits + m.misses for row in models for m in row)

@@ -182,7 +182,7 @@ def test_topk_select(K, B, n, KH, k, lo, hi, max_score):
 
 def test_topk_select_head_major_and_seq_lens(K):
     g = _gen(11)
-    s = _scores(g, 2, 5000, 8, 230, 290, 512)
+    s = _scores(g, 2, 5000, 8, 230, 290)
     lens = torch.tensor([5000, 1234], dtype=torch.int32)
     sh = s.permute(0, 2, 1).contiguous()  # [B, KH, n]
     got = K.topk_select(sh.to(DEV), 99, 512, lens.to(DEV), layout="bhn").cpu().numpy()
@@ -193,7 +193,7 @@ def test_topk_select_head_major_and_seq_lens(K):
 
 def test_topk_relation_to_torch_topk(K):
     # torch.topk may pick other indices among ties; the multiset of kept scores must agree
-    s = _scores(_gen(12), 2, 3000, 4, 240, 272, 512)
+    s = _scores(_gen(12), 2, 3000, 4, 240, 272)
     idx = K.topk_select(s.to(DEV), 300, 512).cpu().long()
     kept = torch.gather(s.permute(0, 2, 1), 2, idx).sort(dim=2).values
     ref = s.permute(0, 2, 1).to(torch.int32).topk(300, dim=2).values.sort(dim=2).values
@@ -361,4 +361,4 @@ def test_cache_append(K):
     assert torch.equal(out[:, :7], a)
     for bi, l in enumerate([7, 9, 30]):
         assert torch.equal(out[bi, l], b[bi, 0])
-    assert out.float().abs().sum() == a.float().abs().sum() + b.float().abs().sum()
+    assert int((out.float().abs().sum(dim=(2, 3)) > 0).sum()) == 3 * 7 + 3   # nothing else was written
