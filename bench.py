@@ -1,0 +1,292 @@
+#!/usr/bin/env python3
+"""Decode-time retrieval benchmark: sparse-decode us/step/layer and achieved HBM GB/s.
+
+A *step* is one decode step of ONE attention layer: hash the new query and key,
+append code + K + V, score every cached code, select the top k per (batch, kv
+head), optionally update the LRU resident table, and attend over the selected
+rows.  Consecutive steps walk round-robin over ``--layers`` independent layer
+states (a real decode token visits every layer once), so no layer finds its
+codes or K/V in L2 from its previous visit.  One HIP graph holds one token
+(= ``layers`` steps plus the delivery of that token's fresh q/k/v from a
+pre-generated pool); replays are timed with the inputs resident in HBM.
+
+Prints ONE JSON line.  ``value`` is microseconds per step (lower is better);
+``roofline`` prices the dominant kernel against the 8 TB/s HBM peak of MI355X
+on its algorithmic bytes; ``cpu_baseline`` is the CPU oracle's cached-codes
+decode step timed on this host on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+CONFIGS = {
+    # name: B, QH, KH, n0, k, dtype, hash, lru slots, default layers, description
+    "c1": dict(B=1, QH=32, KH=32, n0=4096, k=410, dtype="f32", hash="linear", lru=0, layers=32,
+               desc="Llama-2-7B shape, fp32, linear 128x128 Gaussian hash, 90% pruned"),
+    "c2": dict(B=1, QH=32, KH=8, n0=32768, k=655, dtype="bf16", hash="mlp", lru=0, layers=32,
+               desc="Llama-3-8B GQA, bf16, 32k ctx, MLP 128-256-128 hash, 98% pruned"),
+    "c3": dict(B=16, QH=32, KH=8, n0=16384, k=328, dtype="bf16", hash="mlp", lru=1024, layers=32,
+               desc="Llama-3-8B GQA, bf16, batch 16 x 16k ctx, LRU resident buffer 1024, 98% pruned"),
+    "c4": dict(B=1, QH=40, KH=8, n0=131072, k=2622, dtype="bf16", hash="mlp", lru=0, layers=16,
+               desc="Qwen2.5-14B shape, bf16, 128k ctx, 98% pruned"),
+}
+
+
+def algorithmic_bytes(c, n):
+    """Bytes one step of one layer has to move, intermediates excluded."""
+    s = 4 if c["dtype"] == "f32" else 2
+    B, QH, KH, k, d, nbits = c["B"], c["QH"], c["KH"], c["k"], 128, 128
+    if c["hash"] == "mlp":
+        per_head = (128 * 256 + 256 + 256 * 128 + 128) * s
+        w = per_head * (QH + KH)
+    else:
+        w = 128 * 128 * s * (QH if KH == QH else QH + KH)
+    io_new = B * (QH + 2 * KH) * d * s                       # q, k_new, v_new read
+    append = B * KH * (nbits // 8 + 2 * d * s)               # code + K + V written
+    hash_b = w + io_new + append + B * QH * nbits // 8
+    score_b = B * n * KH * nbits // 8 + B * QH * nbits // 8  # codes streamed + q codes
+    attn_b = 2 * B * k * KH * d * s + 2 * B * QH * d * s     # selected K and V rows, q, out
+    lru_b = 0
+    return {"hash": hash_b, "score": score_b, "select": 0, "lru": lru_b, "attn": attn_b,
+            "step": w + B * QH * d * s + B * n * KH * nbits // 8 + 2 * B * k * KH * d * s + B * QH * d * s + append}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--layers", type=int, default=None)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-breakdown", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path shards over (batch, kv head) without any exchange, "
+              "so this build has no multi-GPU figure; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from spotlight_amd import _lib, decode, kernel
+
+    c = dict(CONFIGS[args.config])
+    L = args.layers or c["layers"]
+    steps = args.steps if args.steps is not None else (256 if args.config == "c3" else 1000)
+    warmup = args.warmup if args.warmup is not None else 64
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    dtype = torch.float32 if c["dtype"] == "f32" else torch.bfloat16
+    B, QH, KH, n0, k, d = c["B"], c["QH"], c["KH"], c["n0"], c["k"], 128
+
+    tokens = math.ceil(warmup / L) + math.ceil(steps / L) + 4 + 64   # cache growth incl. the breakdown passes
+    n_cap = (n0 + tokens + 7) // 8 * 8
+
+    cpu_gen = torch.Generator()
+    cpu_gen.manual_seed(0)
+    gpu_gen = torch.Generator(device=dev)
+    gpu_gen.manual_seed(0)
+
+    # per-token inputs for every layer, drawn once; a token's slice is copied in by the graph
+    P = 16
+    pool = [torch.randn((P, L, B, h, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
+            for h in (QH, KH, KH)]
+    cur = [torch.empty((1, L, B, h, d), device=dev, dtype=dtype) for h in (QH, KH, KH)]
+    tok = torch.zeros((1,), dtype=torch.int64, device=dev)
+
+    layers = []
+    for li in range(L):
+        if c["hash"] == "mlp":
+            hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, dev, cpu_gen)
+            hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, dev, cpu_gen)
+        else:
+            hq = decode.HashWeights.random_linear(QH, 128, 128, dtype, dev, cpu_gen)
+            hk = hq if KH == QH else decode.HashWeights.random_linear(KH, 128, 128, dtype, dev, cpu_gen)
+        st = decode.LayerDecodeState(B, QH, KH, d, n_cap, k, hq, hk, dtype=dtype, device=dev,
+                                     lru_slots=c["lru"], inputs=tuple(t[0, li] for t in cur))
+        # prefill in slabs to bound the transient memory of hashing
+        st.seq_lens.zero_()
+        slab = max(1, (1 << 22) // (B * KH))
+        for s0 in range(0, n0, slab):
+            s1 = min(n0, s0 + slab)
+            kk = torch.randn((B, s1 - s0, KH, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
+            vv = torch.randn((B, s1 - s0, KH, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
+            st.keys[:, s0:s1] = kk
+            st.vals[:, s0:s1] = vv
+            kernel.cache_append(st.codes, st.hash_k.hash_rows(kk), start=s0)
+        st.seq_lens.fill_(n0)
+        st.host_len = n0
+        layers.append(st)
+    torch.cuda.synchronize()
+
+    def token_body(n_max):
+        for i in range(3):
+            torch.index_select(pool[i], 0, tok, out=cur[i])
+        tok.add_(1).remainder_(P)
+        for st in layers:
+            st._launch(n_max)
+
+    def capture(fn):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g
+
+    n_max = n0 + tokens
+    token_graph = capture(lambda: token_body(n_max))
+
+    def run_steps(nsteps):
+        full, rem = divmod(nsteps, L)
+        for _ in range(full):
+            token_graph.replay()
+        if rem:  # a partial token: deliver inputs, then the first `rem` layers, eagerly
+            for i in range(3):
+                torch.index_select(pool[i], 0, tok, out=cur[i])
+            tok.add_(1).remainder_(P)
+            for st in layers[:rem]:
+                st._launch(n_max)
+
+    run_steps(warmup)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    run_steps(steps)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = ev0.elapsed_time(ev1)
+    ms_per_step = wall_ms / steps
+    us_per_step = ms_per_step * 1e3
+    n_mid = n0 + (math.ceil(warmup / L) + steps / L / 2)
+    ab = algorithmic_bytes(c, n_mid)
+
+    # ---- per-kernel durations: HIP events around a graph of M launches of one stage, rotating layers
+    kernels = {}
+    dominant = None
+    if not args.no_kernel_breakdown:
+        # equalise lengths (a partial token may have advanced only some layers)
+        M = 4 * L
+        stage_sets = [("hash", _lib.STAGE_HASH), ("score", _lib.STAGE_SCORE),
+                      ("score+select", _lib.STAGE_SCORE | _lib.STAGE_SELECT), ("attn", _lib.STAGE_ATTN)]
+        if c["lru"]:
+            stage_sets.insert(3, ("lru", _lib.STAGE_LRU))
+        raw = {}
+        for name, mask in stage_sets:
+            def body(mask=mask):
+                for j in range(M):
+                    layers[j % L]._launch(n_max, mask)
+            g = capture(body)
+            g.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            raw[name] = e0.elapsed_time(e1) * 1e3 / M
+            del g
+            if name == "score":
+                for st in layers:
+                    st.reset_workspace()
+                torch.cuda.synchronize()
+        raw["select"] = max(raw["score+select"] - raw["score"], 0.0)
+        for name in ("hash", "score", "select", "lru", "attn"):
+            if name in raw:
+                us = raw[name]
+                kernels[name] = {"us": round(us, 3), "algorithmic_bytes": ab[name],
+                                 "gbps": round(ab[name] / us / 1e3, 1) if us > 0 else None}
+        dominant = max((n for n in kernels if kernels[n]["algorithmic_bytes"] > 0), key=lambda n: kernels[n]["us"])
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    if dominant and os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(args.config, {}).get(dominant)
+    roofline = None
+    if dominant:
+        ach = kernels[dominant]["gbps"]
+        roofline = {"kernel": dominant, "bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                    "algorithmic_bytes_per_launch": kernels[dominant]["algorithmic_bytes"],
+                    "us_per_launch": kernels[dominant]["us"]}
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        cpu_baseline = cpu_leg(layers[0], c, budget_s=20.0)
+
+    step_gbps = ab["step"] / us_per_step / 1e3
+    out = {
+        "metric": "sparse-decode us/step/layer (Llama-3-8B GQA, 32k ctx)" if args.config == "c2"
+                  else f"sparse-decode us/step/layer ({args.config})",
+        "value": round(us_per_step, 3), "unit": "us/step/layer", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": c["dtype"], "data": "synthetic",
+        "config": {"workload": f"{args.config}: {c['desc']}", "batch": B, "q_heads": QH, "kv_heads": KH,
+                   "head_dim": d, "context": n0, "k": k, "code_bits": 128, "hash": c["hash"],
+                   "lru_slots": c["lru"], "layers_rotated": L, "graph": "one HIP graph per token"},
+        "gpu_event_ms_per_step": round(gpu_ms / steps, 6),
+        "hbm_gbps": round(step_gbps, 1), "hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes_per_step": int(ab["step"]),
+        "tokens_per_s": round(B / (ms_per_step * 1e-3 * L), 2), "tokens_per_s_layers": L,
+        "kernels": kernels, "roofline": roofline, "cpu_baseline": cpu_baseline,
+    }
+    print(json.dumps(out), flush=True)
+
+
+def cpu_leg(st, c, budget_s):
+    """The oracle's cached-codes decode step (hash q -> pack -> XOR/popcount -> stable
+    top-k -> gather -> softmax attention) on this host, on layer 0's real cache."""
+    import numpy as np
+    import torch
+
+    from oracle import spotlight_oracle as orc
+
+    n = int(st.seq_lens.max().item())
+    B, QH, KH, k = st.B, st.QH, st.KH, st.k
+    codes = st.codes[:, :n].cpu().numpy()
+    keys, vals = st.keys[:, :n].cpu(), st.vals[:, :n].cpu()
+    hq = st.hash_q
+    ws = [(hq.w1.cpu()[None], (hq.b1.cpu() if hq.b1 is not None else torch.zeros(QH, hq.d_hid, dtype=hq.w1.dtype))[None, :, None])]
+    if hq.w2 is not None:
+        ws.append((hq.w2.cpu()[None], hq.b2.cpu()[None, :, None]))
+    g = torch.Generator()
+    g.manual_seed(1)
+    bidx = torch.arange(B)[:, None, None]
+    hidx = torch.arange(KH)[None, :, None]
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
+        q = torch.randn(B, QH, 128, generator=g).to(st.dtype)
+        t0 = time.perf_counter()
+        pre = orc.mlp_hash_torch(q.unsqueeze(2), ws, hq.residue).squeeze(2)
+        q_code = orc.pack_sign_u32(pre.float().numpy())[:, None]
+        score = orc.hamming_score_u32(q_code, codes, st.head_map)
+        idx = orc.topk_stable(score, k)
+        ti = torch.from_numpy(idx).long()
+        ks = keys[bidx, ti, hidx].float()            # [B,KH,k,d]
+        vs = vals[bidx, ti, hidx].float()
+        qg = q.float().view(B, KH, QH // KH, 128)
+        p = torch.softmax(torch.einsum("bhgd,bhkd->bhgk", qg, ks) / math.sqrt(128), dim=-1)
+        _ = torch.einsum("bhgk,bhkd->bhgd", p, vs)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(med * 1e6, 1), "unit": "us/step/layer", "cores": torch.get_num_threads(),
+            "kind": "port", "host_cpus": os.cpu_count(),
+            "sample": f"{len(times)} decode steps of one layer at n={n} (median), numpy/torch CPU restatement "
+                      "with cached key codes"}
+
+
+if __name__ == "__main__":
+    main()

@@ -237,6 +237,16 @@ typedef struct {
 size_t sl_decode_workspace_bytes(const sl_decode_params *p);
 int sl_decode_step(const sl_decode_params *p, void *stream);
 
+/* The same step restricted to a subset of its kernels, for profiling one
+ * kernel at a time on real shapes.  Lengths and the step counter only advance
+ * when every stage runs; running SCORE without SELECT leaves counts in the
+ * workspace histogram (clear it with sl_workspace_init before a real step). */
+enum {
+    SL_STAGE_HASH = 1, SL_STAGE_SCORE = 2, SL_STAGE_SELECT = 4, SL_STAGE_LRU = 8, SL_STAGE_ATTN = 16,
+    SL_STAGE_ALL = 31
+};
+int sl_decode_stages(const sl_decode_params *p, int stages, void *stream);
+
 /* Zero-fills a workspace with a kernel (safe inside a captured HIP graph). */
 int sl_workspace_init(void *ws, size_t ws_bytes, void *stream);
 

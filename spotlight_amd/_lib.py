@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libspotlight_hip.so")
 
 SL_F32, SL_BF16, SL_F16 = 0, 1, 2
 SL_HEADMAP_INTERLEAVED, SL_HEADMAP_BLOCKED = 0, 1
+STAGE_HASH, STAGE_SCORE, STAGE_SELECT, STAGE_LRU, STAGE_ATTN, STAGE_ALL = 1, 2, 4, 8, 16, 31
 
 c_void_p, c_int, c_int64, c_size_t, c_float, c_uint32 = (
     C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float, C.c_uint32)
@@ -58,6 +59,7 @@ SIGNATURES = {
     "sl_sparse_gqa_attn": (c_int, [c_void_p] * 5 + [c_int] * 6 + [c_int64] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),
     "sl_decode_workspace_bytes": (c_size_t, [C.POINTER(DecodeParams)]),
     "sl_decode_step": (c_int, [C.POINTER(DecodeParams), c_void_p]),
+    "sl_decode_stages": (c_int, [C.POINTER(DecodeParams), c_int, c_void_p]),
     "sl_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
 }
 

@@ -40,20 +40,26 @@ def build_library(verbose: bool = True, jobs: int = 4) -> str:
     objdir = os.path.join(CSRC, "build")
     os.makedirs(objdir, exist_ok=True)
 
-    def compile_one(src: str) -> str:
-        obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    def run(cmd) -> None:
         if verbose:
             print(" ".join(cmd), flush=True)
-        subprocess.run(cmd, check=True)
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        # the host pass does not know the gfx feature named in HIPCC_FLAGS and says so; harmless
+        noise = "'-packed-fp32-ops' is not a recognized feature"
+        out = "\n".join(l for l in res.stdout.splitlines() if noise not in l)
+        if out.strip():
+            print(out, flush=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed ({res.returncode}): {' '.join(cmd)}")
+
+    def compile_one(src: str) -> str:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        run([hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(compile_one, SOURCES))
-    cmd = [hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", LIB_PATH]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
+    run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", LIB_PATH])
     return LIB_PATH
 
 

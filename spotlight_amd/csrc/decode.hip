@@ -91,7 +91,12 @@ extern "C" size_t sl_decode_workspace_bytes(const sl_decode_params *p) {
 }
 
 extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
+    return sl_decode_stages(pp, SL_STAGE_ALL, stream);
+}
+
+extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *stream) {
     SL_REQUIRE(pp, SL_ERR_NULL);
+    SL_REQUIRE((stages & ~SL_STAGE_ALL) == 0, SL_ERR_SHAPE);
     const sl_decode_params &p = *pp;
     int rc = validate(p);
     if (rc != SL_OK) return rc;
@@ -123,8 +128,10 @@ extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
     sk.copy_src[0] = p.k_new; sk.copy_dst[0] = p.keys;
     sk.copy_src[1] = p.v_new; sk.copy_dst[1] = p.vals;
     sk.copy_dst_stride_b = p.n_cap * p.KH * p.d; sk.copy_dst_stride_n = static_cast<int64_t>(p.KH) * p.d;
-    rc = sl_hash_launch(ha, ws + L.hash, L.attn - L.hash, s);
-    if (rc != SL_OK) return rc;
+    if (stages & SL_STAGE_HASH) {
+        rc = sl_hash_launch(ha, ws + L.hash, L.attn - L.hash, s);
+        if (rc != SL_OK) return rc;
+    }
 
     // 2. score seq_lens[b] + 1 rows
     hamming_args sa{};
@@ -132,22 +139,27 @@ extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
     sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
     sa.n_bins = G * p.nbits + 1; sa.len_bias = 1; sa.n = p.n_max; sa.n_cap = p.n_cap;
     sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
-    rc = sl_hamming_launch(sa, true, s);
-    if (rc != SL_OK) return rc;
+    if (stages & SL_STAGE_SCORE) {
+        rc = sl_hamming_launch(sa, true, s);
+        if (rc != SL_OK) return rc;
+    }
 
     // 3. select
     select_args ta{};
     ta.score = score; ta.hist = hist; ta.idx = p.idx; ta.seq_lens = p.seq_lens;
     ta.B = p.B; ta.KH = p.KH; ta.k = p.k; ta.n_bins = sa.n_bins; ta.len_bias = 1; ta.n = p.n_max;
     ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
-    rc = sl_select_launch(ta, s);
-    if (rc != SL_OK) return rc;
+    if (stages & SL_STAGE_SELECT) {
+        rc = sl_select_launch(ta, s);
+        if (rc != SL_OK) return rc;
+    }
 
     // 4. optional LRU, 5. attention
     attn_args aa{};
     aa.q = p.q; aa.out = p.out; aa.dtype = p.dtype; aa.B = p.B; aa.QH = p.QH; aa.KH = p.KH; aa.k = p.k;
     aa.rows = 0; aa.scale = 0.f; aa.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
-    aa.bump_lens = p.seq_lens; aa.bump_step = p.step_counter;
+    const bool whole = stages == SL_STAGE_ALL;  // lengths only advance on a complete step
+    aa.bump_lens = whole ? p.seq_lens : nullptr; aa.bump_step = whole ? p.step_counter : nullptr;
     if (p.lru_C > 0) {
         SL_REQUIRE(p.k + 1 <= p.lru_C && p.lru_C <= LRU_MAX_SLOTS, SL_ERR_UNSUPPORTED);
         lru_args la{};
@@ -156,8 +168,10 @@ extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
         la.slots_out = p.slots_out; la.stats = p.lru_stats; la.stamp_dev = p.step_counter; la.stamp = 1;
         la.dtype = p.dtype; la.B = p.B; la.KH = p.KH; la.d = p.d; la.k = p.k; la.C = p.lru_C;
         la.map_cap = p.lru_map_cap; la.kv_stride_b = p.n_cap * p.KH * p.d;
-        rc = sl_lru_launch(la, s);
-        if (rc != SL_OK) return rc;
+        if (stages & SL_STAGE_LRU) {
+            rc = sl_lru_launch(la, s);
+            if (rc != SL_OK) return rc;
+        }
         aa.keys = p.k_res; aa.vals = p.v_res; aa.idx = p.slots_out;
         aa.kv_stride_b = static_cast<int64_t>(p.KH) * p.lru_C * p.d;
         aa.kv_stride_h = static_cast<int64_t>(p.lru_C) * p.d;
@@ -167,5 +181,6 @@ extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
         aa.kv_stride_b = p.n_cap * p.KH * p.d; aa.kv_stride_h = p.d;
         aa.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
     }
+    if (!(stages & SL_STAGE_ATTN)) return SL_OK;
     return sl_attn_launch(aa, ws + L.attn, L.total - L.attn, s);
 }

@@ -93,7 +93,7 @@ class HashWeights:
 class LayerDecodeState:
     def __init__(self, batch_size: int, num_heads: int, num_kv_heads: int, head_dim: int, n_cap: int, k: int,
                  hash_q: HashWeights, hash_k: HashWeights, dtype=torch.bfloat16, device="cuda",
-                 head_map: str = "blocked", lru_slots: int = 0):
+                 head_map: str = "blocked", lru_slots: int = 0, inputs=None):
         assert head_dim == 128, "the attention kernel covers head_dim 128"
         assert n_cap % 8 == 0, "n_cap must be a multiple of 8"
         assert hash_q.nbits == hash_k.nbits and hash_q.n_layers == hash_k.n_layers
@@ -111,9 +111,13 @@ class LayerDecodeState:
         self.vals = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=dev)
         self.seq_lens = torch.zeros((B,), dtype=torch.int32, device=dev)
         self.step_counter = torch.zeros((1,), dtype=torch.int32, device=dev)
-        self.q_in = torch.zeros((B, QH, d), dtype=dtype, device=dev)
-        self.k_in = torch.zeros((B, KH, d), dtype=dtype, device=dev)
-        self.v_in = torch.zeros((B, KH, d), dtype=dtype, device=dev)
+        if inputs is None:  # the step's inputs are read from these buffers
+            inputs = (torch.zeros((B, QH, d), dtype=dtype, device=dev),
+                      torch.zeros((B, KH, d), dtype=dtype, device=dev),
+                      torch.zeros((B, KH, d), dtype=dtype, device=dev))
+        self.q_in, self.k_in, self.v_in = inputs
+        assert self.q_in.shape == (B, QH, d) and self.k_in.shape == (B, KH, d) and self.v_in.shape == (B, KH, d)
+        assert all(t.is_contiguous() and t.dtype == dtype for t in inputs)
         self.out = torch.zeros((B, QH, d), dtype=dtype, device=dev)
         self.idx = torch.full((B, KH, k), -1, dtype=torch.int32, device=dev)
         self.host_len = 0  # upper bound of seq_lens, tracked on the host for grid sizing
@@ -178,20 +182,35 @@ class LayerDecodeState:
         self.host_len = n0
 
     # -- decode ------------------------------------------------------------------
-    def _launch(self, n_max: int) -> None:
+    def _launch(self, n_max: int, stages: int = _lib.STAGE_ALL) -> None:
         if n_max > self.n_cap:
             raise RuntimeError(f"cache capacity {self.n_cap} exceeded")
         self.params.n_max = n_max
-        _lib.check(_L.sl_decode_step(C.byref(self.params), torch.cuda.current_stream().cuda_stream),
-                   "sl_decode_step")
+        _lib.check(_L.sl_decode_stages(C.byref(self.params), stages, torch.cuda.current_stream().cuda_stream),
+                   "sl_decode_stages")
+
+    def launch_stages(self, stages: int) -> None:
+        """Enqueue a subset of the step's kernels on the current inputs (profiling
+        aid; lengths do not advance).  After SCORE without SELECT call
+        ``reset_workspace`` before the next real step."""
+        with torch.cuda.device(self.device):
+            self._launch(self.host_len + 1, stages)
+
+    def reset_workspace(self) -> None:
+        with torch.cuda.device(self.device):
+            _lib.check(_L.sl_workspace_init(self.ws.data_ptr(), self.ws.numel(),
+                                            torch.cuda.current_stream().cuda_stream), "sl_workspace_init")
 
     def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor) -> torch.Tensor:
         """One decode step: q [B,QH,d], k_new/v_new [B,KH,d] (post-RoPE).
         Returns the attention output [B,QH,d] (a buffer reused by the next step)."""
         with torch.cuda.device(self.device):
-            self.q_in.copy_(q)
-            self.k_in.copy_(k_new)
-            self.v_in.copy_(v_new)
+            if q is not self.q_in:
+                self.q_in.copy_(q)
+            if k_new is not self.k_in:
+                self.k_in.copy_(k_new)
+            if v_new is not self.v_in:
+                self.v_in.copy_(v_new)
             self._launch(self.host_len + 1)
         self.host_len += 1
         return self.out
