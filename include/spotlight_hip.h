@@ -72,16 +72,12 @@ int sl_pack_sign_u8(const void *x, int dtype, uint8_t *out, int64_t n_bytes, voi
  * where the reference's torch expression rounds it; accumulation is fp32.
  * code_row[b] (may be NULL, then 0) is added to the code row index, in units
  * of code_stride_n, so that a key code lands in cache row seq_len[b].
- * ws: sl_hash_workspace_bytes(B, H, d_hid, nbits) bytes, zeroed once with
- * sl_workspace_init(); its first 16 KiB (arrival tickets, H <= 4096) are left
- * zeroed, so one workspace can serve calls of any shape it is big enough for. */
-size_t sl_hash_workspace_bytes(int B, int H, int d_hid, int nbits);
+ * d_in == 128; d_hid in {64, 128, 256, 512}; two layers need nbits == 128. */
 int sl_hash_mlp_pack(const void *x, const void *w1, const void *b1, const void *w2,
                      const void *b2, uint32_t *codes, int dtype, int n_layers, int B,
                      int H, int d_in, int d_hid, int nbits, int residue,
                      int64_t x_stride_b, int64_t code_stride_b, int64_t code_stride_h,
-                     int64_t code_stride_n, const int32_t *code_row, void *ws,
-                     size_t ws_bytes, void *stream);
+                     int64_t code_stride_n, const int32_t *code_row, void *stream);
 
 /* ---- (b) Hamming scorer -------------------------------------------------- */
 
@@ -115,9 +111,9 @@ int sl_hamming_score_u8(const uint8_t *q, const uint8_t *k, uint8_t *out, int BH
  *          lowest token index, listed in ascending token order; when fewer
  *          than k tokens exist the tail is filled with -1.
  * seq_lens (may be NULL): per-batch token count on the device (<= n).
- * ws: sl_topk_workspace_bytes(B, KH, max_score), zeroed once with
- * sl_workspace_init(); left zeroed. */
-size_t sl_topk_workspace_bytes(int B, int KH, int max_score);
+ * ws: sl_topk_workspace_bytes(B, KH, max_score, n) bytes of scratch; it needs
+ * no initialisation. */
+size_t sl_topk_workspace_bytes(int B, int KH, int max_score, int64_t n);
 int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
                    int32_t *idx, int B, int64_t n, int KH, int k, int max_score,
                    const int32_t *seq_lens, void *ws, size_t ws_bytes, void *stream);
@@ -239,8 +235,8 @@ int sl_decode_step(const sl_decode_params *p, void *stream);
 
 /* The same step restricted to a subset of its kernels, for profiling one
  * kernel at a time on real shapes.  Lengths and the step counter only advance
- * when every stage runs; running SCORE without SELECT leaves counts in the
- * workspace histogram (clear it with sl_workspace_init before a real step). */
+ * when every stage runs.  HASH also clears the score histogram, so SCORE
+ * without a preceding HASH keeps adding to it. */
 enum {
     SL_STAGE_HASH = 1, SL_STAGE_SCORE = 2, SL_STAGE_SELECT = 4, SL_STAGE_LRU = 8, SL_STAGE_ATTN = 16,
     SL_STAGE_ALL = 31

@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libspotlight_hip.so")
+# SPOTLIGHT_HIP_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("SPOTLIGHT_HIP_LIB") or os.path.join(_HERE, "libspotlight_hip.so")
 
 SL_F32, SL_BF16, SL_F16 = 0, 1, 2
 SL_HEADMAP_INTERLEAVED, SL_HEADMAP_BLOCKED = 0, 1
@@ -45,11 +46,10 @@ SIGNATURES = {
     "sl_version": (c_int, []),
     "sl_pack_sign_u32": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "sl_pack_sign_u8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
-    "sl_hash_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
-    "sl_hash_mlp_pack": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_int64] * 4 + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sl_hash_mlp_pack": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_int64] * 4 + [c_void_p, c_void_p]),
     "sl_hamming_score": (c_int, [c_void_p] * 3 + [c_int, c_int64, c_int, c_int, c_int] + [c_int64] * 3 + [c_int, c_void_p, c_void_p]),
     "sl_hamming_score_u8": (c_int, [c_void_p] * 3 + [c_int, c_int64, c_int, c_void_p]),
-    "sl_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "sl_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int64]),
     "sl_topk_select": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_int, c_int, c_int,
                                c_void_p, c_void_p, c_size_t, c_void_p]),
     "sl_gather_kv": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64, c_void_p]),

@@ -12,7 +12,7 @@ struct attn_args {
     int32_t *bump_lens;     // optional [B]: incremented once per call
     uint32_t *bump_step;    // optional [1]: incremented once per call
     int dtype, B, QH, KH, k;
-    int rows;               // rows per workgroup: 16, 32 or 64 (0 = choose)
+    int rows;               // ranks per workgroup, a multiple of 64 (0 = choose)
     int64_t q_stride_b, kv_stride_b, kv_stride_n, kv_stride_h;
     float scale;
 };

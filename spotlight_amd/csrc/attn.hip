@@ -1,36 +1,44 @@
 // (e) gather-based sparse GQA decode attention.
 //
-// The k selected rows of a (batch, kv head) are split into runs of `rows`
-// consecutive ranks; one workgroup of 4 waves handles one run.  A K or V row
-// of 128 elements is read by 16 lanes with one 16-byte load each (two for
-// fp32), so a wave covers 4 rows per load and the workgroup 16; every K and V
-// load of the run is issued before the first dot product (V addresses do not
-// depend on the scores), which makes the run one memory round trip.  Each
-// lane keeps its 8-element slice of the G query rows in registers, dots it
-// with the K slice, and a 16-lane DPP reduction completes the score; the G
-// heads of the group reuse every K/V byte from registers, so nothing is
-// staged twice.  Softmax over the run is done in LDS, the G x 128 partial
-// output with its (max, sum) goes to the workspace, and the last workgroup of
-// a (b, kv head) to arrive merges the runs by log-sum-exp in run order, so the
-// result does not depend on arrival order.
+// The step is latency bound (a few MB per layer), so the kernel is organised
+// around memory round trips rather than around occupancy:
+//   * the k selected rows of a (batch, kv head) are cut into at most
+//     AT_MAX_SPLITS runs of `rows` consecutive ranks, one workgroup of 4 waves
+//     per run; the run's row numbers are fetched into LDS in one go;
+//   * a K or V row of 128 elements is read by 16 lanes with one 16-byte load
+//     each (two for fp32), so a wave covers 4 rows per load and the workgroup
+//     16; AT_U such row groups -- K and V alike, V addresses do not depend on
+//     the scores -- are in flight before the first dot product;
+//   * each 16-lane group keeps its 8-element slice of the G query rows in
+//     registers and carries its own running softmax state (max, sum, 8
+//     accumulators per query head), so the G heads of the group reuse every
+//     K/V byte from registers and there is no barrier inside the row loop;
+//   * the 16 lane-group states are merged with shuffles and LDS; a run's
+//     (acc, max, sum) goes to the workspace through device-coherent stores;
+//     the last workgroup of a (b, kv head) to arrive loads all runs'
+//     partials at once (one round trip) and merges them in run order, so
+//     the result does not depend on arrival order.
 #include "attn.h"
 
 namespace {
 
 constexpr int AT_THREADS = 256;
 constexpr int AT_D = 128;
-constexpr int AT_PART = AT_D + 2;  // acc[128], m, l
+constexpr int AT_PART = AT_D + 2;    // acc[128], m, l
+constexpr int AT_U = 4;              // row groups in flight per iteration (64 rows per workgroup)
+constexpr int AT_ITER_ROWS = 16 * AT_U;
+constexpr int AT_MAX_SPLITS = 16;    // runs per (b, kv head): the merge loads them all at once
+constexpr int AT_MAX_ROWS = 1024;    // rows per run (LDS row-number buffer)
 // The arrival tickets sit in a fixed-size head of the workspace so that the
 // partials of a call with other shapes can never land on them: the tickets are
 // the only part that has to stay zero between calls.
 constexpr size_t AT_COUNTER_BYTES = 64 * 1024;
 
-template <typename T, int G, int STEPS>
+template <typename T, int G>
 __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
-    constexpr int R = 16 * STEPS;
-    __shared__ float s_p[G][R];
-    __shared__ float s_m[G], s_l[G];
-    __shared__ float s_red[4][G][AT_D];
+    __shared__ int s_row[AT_MAX_ROWS];
+    __shared__ float s_m[4][G], s_l[4][G];
+    __shared__ __align__(16) float s_acc[4][G][AT_D];
     __shared__ int s_last;
 
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -39,6 +47,11 @@ __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
     const int wave = tid >> 6, lane = tid & 63;
     const int sub = lane & 15;            // which 8-element slice of the row
     const int rslot = wave * 4 + (lane >> 4);
+
+    const int r_lo = split * a.rows;
+    const int r_hi = r_lo + a.rows < a.k ? r_lo + a.rows : a.k;
+    const int32_t *idx = a.idx + (static_cast<int64_t>(b) * a.KH + h) * a.k;
+    for (int i = tid; i < a.rows; i += AT_THREADS) s_row[i] = r_lo + i < r_hi ? idx[r_lo + i] : -1;
 
     const T *qb = static_cast<const T *>(a.q) + static_cast<int64_t>(b) * a.q_stride_b +
                   static_cast<int64_t>(h) * G * AT_D + sub * 8;
@@ -49,192 +62,191 @@ __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) qf[g][j] *= a.scale;
     }
-
-    const int32_t *idx = a.idx + (static_cast<int64_t>(b) * a.KH + h) * a.k;
     const T *kb = static_cast<const T *>(a.keys) + static_cast<int64_t>(b) * a.kv_stride_b +
                   static_cast<int64_t>(h) * a.kv_stride_h + sub * 8;
     const T *vb = static_cast<const T *>(a.vals) + static_cast<int64_t>(b) * a.kv_stride_b +
                   static_cast<int64_t>(h) * a.kv_stride_h + sub * 8;
 
-    int row[STEPS];
+    float m[G], l[G], acc[G][8];
 #pragma unroll
-    for (int st = 0; st < STEPS; ++st) {
-        const int rank = split * R + st * 16 + rslot;
-        row[st] = rank < a.k ? idx[rank] : -1;
-    }
-    float kf[STEPS][8], vf[STEPS][8];
-#pragma unroll
-    for (int st = 0; st < STEPS; ++st) {
-        if (row[st] >= 0) {
-            load8<T>(kb + static_cast<int64_t>(row[st]) * a.kv_stride_n, kf[st]);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) kf[st][j] = 0.f;
-        }
-    }
-#pragma unroll
-    for (int st = 0; st < STEPS; ++st) {
-        if (row[st] >= 0) {
-            load8<T>(vb + static_cast<int64_t>(row[st]) * a.kv_stride_n, vf[st]);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) vf[st][j] = 0.f;
-        }
-    }
-
-    // scores of the run
-#pragma unroll
-    for (int st = 0; st < STEPS; ++st) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            float d = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) d = fmaf(qf[g][j], kf[st][j], d);
-            d = row16_sum(d);
-            if (sub == 0) s_p[g][st * 16 + rslot] = row[st] >= 0 ? d : -INFINITY;
-        }
-    }
-    __syncthreads();
-
-    // softmax statistics of the run: wave w takes heads w, w+4, ...
-    for (int g = wave; g < G; g += 4) {
-        float m = -INFINITY;
-        for (int e = lane; e < R; e += 64) m = fmaxf(m, s_p[g][e]);
-        m = wave_max(m);
-        float l = 0.f;
-        for (int e = lane; e < R; e += 64) {
-            const float p = m == -INFINITY ? 0.f : __expf(s_p[g][e] - m);
-            s_p[g][e] = p;
-            l += p;
-        }
-        l = wave_sum(l);
-        if (lane == 0) { s_m[g] = m; s_l[g] = l; }
-    }
-    __syncthreads();
-
-    // weighted sum of the V rows
-    float acc[G][8];
-#pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY;
+        l[g] = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[g][j] = 0.f;
+    }
+    __syncthreads();
+
+    for (int base = 0; base < a.rows; base += AT_ITER_ROWS) {
+        int row[AT_U];
+        float kf[AT_U][8], vf[AT_U][8];
 #pragma unroll
-    for (int st = 0; st < STEPS; ++st)
+        for (int u = 0; u < AT_U; ++u) row[u] = s_row[base + u * 16 + rslot];
+        // unconditional loads (an unused slot re-reads row 0 and is masked below):
+        // no branch sits between the 2 * AT_U loads
+#pragma unroll
+        for (int u = 0; u < AT_U; ++u)
+            load8<T>(kb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n, kf[u]);
+#pragma unroll
+        for (int u = 0; u < AT_U; ++u)
+            load8<T>(vb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n, vf[u]);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            const float p = s_p[g][st * 16 + rslot];
+            float s[AT_U];
+            float mn = m[g];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[g][j] = fmaf(p, vf[st][j], acc[g][j]);
+            for (int u = 0; u < AT_U; ++u) {
+                float d = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) d = fmaf(qf[g][j], kf[u][j], d);
+                d = row16_sum(d);
+                s[u] = row[u] >= 0 ? d : -INFINITY;
+                mn = fmaxf(mn, s[u]);
+            }
+            if (mn == -INFINITY) continue;  // nothing seen yet (uniform within the 16-lane group)
+            const float sc = __expf(m[g] - mn);  // exp(-inf) = 0 on the first rows
+            float p[AT_U], ps = 0.f;
+#pragma unroll
+            for (int u = 0; u < AT_U; ++u) {
+                p[u] = __expf(s[u] - mn);
+                ps += p[u];
+            }
+            l[g] = fmaf(l[g], sc, ps);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float t = acc[g][j] * sc;
+#pragma unroll
+                for (int u = 0; u < AT_U; ++u) t = fmaf(p[u], vf[u][j], t);
+                acc[g][j] = t;
+            }
+            m[g] = mn;
         }
+    }
+
+    // merge the 4 lane groups of the wave, then the 4 waves
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int g = 0; g < G; ++g) {
+        float mw = fmaxf(m[g], __shfl_xor(m[g], 16, 64));
+        mw = fmaxf(mw, __shfl_xor(mw, 32, 64));
+        const float sc = mw == -INFINITY ? 0.f : __expf(m[g] - mw);
+        float lw = l[g] * sc;
+        lw += __shfl_xor(lw, 16, 64);
+        lw += __shfl_xor(lw, 32, 64);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            float v = acc[g][j];
+            float v = acc[g][j] * sc;
             v += __shfl_xor(v, 16, 64);
             v += __shfl_xor(v, 32, 64);
-            if (lane < 16) s_red[wave][g][sub * 8 + j] = v;
+            acc[g][j] = v;
         }
+        if (lane < 16) {
+            float4 *dst = reinterpret_cast<float4 *>(&s_acc[wave][g][sub * 8]);
+            dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+            dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+            if (sub == 0) { s_m[wave][g] = mw; s_l[wave][g] = lw; }
+        }
+    }
     __syncthreads();
 
     const int bh = b * a.KH + h;
-    if (S == 1) {
-        T *ob = static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.QH + static_cast<int64_t>(h) * G) * AT_D;
-        for (int e = tid; e < G * AT_D; e += AT_THREADS) {
-            const int g = e / AT_D, c = e % AT_D;
-            const float o = s_red[0][g][c] + s_red[1][g][c] + s_red[2][g][c] + s_red[3][g][c];
-            const float l = s_l[g];
-            ob[e] = from_f32<T>(l > 0.f ? o / l : 0.f);
+    T *ob = static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.QH + static_cast<int64_t>(h) * G) * AT_D;
+    float *part = a.part + (static_cast<int64_t>(bh) * S + split) * G * AT_PART;
+    for (int e = tid; e < G * AT_D; e += AT_THREADS) {
+        const int g = e / AT_D, c = e % AT_D;
+        float M = fmaxf(fmaxf(s_m[0][g], s_m[1][g]), fmaxf(s_m[2][g], s_m[3][g]));
+        float O = 0.f, L = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float sc = M == -INFINITY ? 0.f : __expf(s_m[w][g] - M);
+            O = fmaf(s_acc[w][g][c], sc, O);
+            L = fmaf(s_l[w][g], sc, L);
         }
+        if (S == 1) {
+            ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
+        } else {
+            st_agent(part + g * AT_PART + c, O);
+            if (c == 0) {
+                st_agent(part + g * AT_PART + AT_D, M);
+                st_agent(part + g * AT_PART + AT_D + 1, L);
+            }
+        }
+    }
+    if (S == 1) {
         if (tid == 0) {
             if (a.bump_lens && h == 0) a.bump_lens[b] += 1;
             if (a.bump_step && h == 0 && b == 0) a.bump_step[0] += 1;
         }
         return;
     }
-
-    float *part = a.part + (static_cast<int64_t>(bh) * S + split) * G * AT_PART;
-    for (int e = tid; e < G * AT_D; e += AT_THREADS) {
-        const int g = e / AT_D, c = e % AT_D;
-        part[g * AT_PART + c] = s_red[0][g][c] + s_red[1][g][c] + s_red[2][g][c] + s_red[3][g][c];
-    }
-    if (tid < G) {
-        part[tid * AT_PART + AT_D] = s_m[tid];
-        part[tid * AT_PART + AT_D + 1] = s_l[tid];
-    }
-    __threadfence();
+    publish_wait();
     __syncthreads();
-    if (tid == 0) {
-        const uint32_t ticket = __hip_atomic_fetch_add(&a.counter[bh], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = ticket == static_cast<uint32_t>(S - 1);
-    }
+    if (tid == 0) s_last = arrive_last(&a.counter[bh], static_cast<uint32_t>(S));
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
 
-    // merge the S runs in run order
+    // merge the S runs by log-sum-exp: every partial this lane needs is loaded at once
     const float *pb = a.part + static_cast<int64_t>(bh) * S * G * AT_PART;
-    T *ob = static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.QH + static_cast<int64_t>(h) * G) * AT_D;
     for (int e = tid; e < G * AT_D; e += AT_THREADS) {
         const int g = e / AT_D, c = e % AT_D;
-        float M = -INFINITY;
-        for (int s = 0; s < S; ++s) M = fmaxf(M, pb[(static_cast<int64_t>(s) * G + g) * AT_PART + AT_D]);
-        float L = 0.f, O = 0.f;
-        for (int s = 0; s < S; ++s) {
+        float pm[AT_MAX_SPLITS], pl[AT_MAX_SPLITS], pa[AT_MAX_SPLITS];
+#pragma unroll
+        for (int s = 0; s < AT_MAX_SPLITS; ++s) {
             const float *ps = pb + (static_cast<int64_t>(s) * G + g) * AT_PART;
-            const float m = ps[AT_D];
-            const float w = m == -INFINITY ? 0.f : __expf(m - M);
-            L = fmaf(ps[AT_D + 1], w, L);
-            O = fmaf(ps[c], w, O);
+            pm[s] = s < S ? ld_agent(ps + AT_D) : -INFINITY;
+            pl[s] = s < S ? ld_agent(ps + AT_D + 1) : 0.f;
+            pa[s] = s < S ? ld_agent(ps + c) : 0.f;
+        }
+        float M = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < AT_MAX_SPLITS; ++s) M = fmaxf(M, pm[s]);
+        float L = 0.f, O = 0.f;
+#pragma unroll
+        for (int s = 0; s < AT_MAX_SPLITS; ++s) {
+            const float w = pm[s] == -INFINITY ? 0.f : __expf(pm[s] - M);
+            L = fmaf(pl[s], w, L);
+            O = fmaf(pa[s], w, O);
         }
         ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
     }
     if (tid == 0) {
-        a.counter[bh] = 0;
+        st_agent(&a.counter[bh], 0u);
         if (a.bump_lens && h == 0) a.bump_lens[b] += 1;
         if (a.bump_step && h == 0 && b == 0) a.bump_step[0] += 1;
     }
 }
 
-template <typename T, int G, int STEPS>
-int launch(const attn_args &a, hipStream_t s) {
-    const int R = 16 * STEPS;
-    const int S = (a.k + R - 1) / R;
-    sparse_attn_kernel<T, G, STEPS><<<dim3(S, a.KH, a.B), dim3(AT_THREADS), 0, s>>>(a);
-    return sl_check_launch();
-}
-
 template <typename T, int G>
-int dispatch_rows(const attn_args &a, hipStream_t s) {
-    switch (a.rows) {
-        case 16: return launch<T, G, 1>(a, s);
-        case 32: return launch<T, G, 2>(a, s);
-        case 64: return launch<T, G, 4>(a, s);
-        default: return SL_ERR_UNSUPPORTED;
-    }
+int launch(const attn_args &a, hipStream_t s) {
+    const int S = (a.k + a.rows - 1) / a.rows;
+    sparse_attn_kernel<T, G><<<dim3(S, a.KH, a.B), dim3(AT_THREADS), 0, s>>>(a);
+    return sl_check_launch();
 }
 
 template <typename T>
 int dispatch_g(const attn_args &a, hipStream_t s) {
     switch (a.QH / a.KH) {
-        case 1: return dispatch_rows<T, 1>(a, s);
-        case 2: return dispatch_rows<T, 2>(a, s);
-        case 4: return dispatch_rows<T, 4>(a, s);
-        case 5: return dispatch_rows<T, 5>(a, s);
-        case 7: return dispatch_rows<T, 7>(a, s);
-        case 8: return dispatch_rows<T, 8>(a, s);
+        case 1: return launch<T, 1>(a, s);
+        case 2: return launch<T, 2>(a, s);
+        case 3: return launch<T, 3>(a, s);
+        case 4: return launch<T, 4>(a, s);
+        case 5: return launch<T, 5>(a, s);
+        case 6: return launch<T, 6>(a, s);
+        case 7: return launch<T, 7>(a, s);
+        case 8: return launch<T, 8>(a, s);
         default: return SL_ERR_UNSUPPORTED;
     }
 }
 
-// Rows per workgroup: the largest run that still leaves about two workgroups
-// per compute unit, so that short selections spread over the whole chip and
-// long ones keep the merge small.
+// Rows per run: about one workgroup per compute unit over the whole launch,
+// never more than AT_MAX_SPLITS runs per (b, kv head), whole 64-row iterations.
 int pick_rows(int B, int KH, int k) {
     const int64_t bh = static_cast<int64_t>(B) * KH;
-    for (int r = 64; r > 16; r >>= 1)
-        if (bh * ((k + r - 1) / r) >= 512) return r;
-    return 16;
+    int64_t want = (256 + bh - 1) / bh;
+    if (want < 1) want = 1;
+    if (want > AT_MAX_SPLITS) want = AT_MAX_SPLITS;
+    int rows = static_cast<int>((k + want - 1) / want);
+    rows = (rows + AT_ITER_ROWS - 1) / AT_ITER_ROWS * AT_ITER_ROWS;
+    return rows;
 }
 
 }  // namespace
@@ -242,9 +254,8 @@ int pick_rows(int B, int KH, int k) {
 size_t sl_attn_ws_bytes(int B, int QH, int KH, int k) {
     if (B <= 0 || QH <= 0 || KH <= 0 || k <= 0) return 0;
     const size_t bh = static_cast<size_t>(B) * KH;
-    const size_t S = (static_cast<size_t>(k) + 15) / 16;
     const size_t G = static_cast<size_t>(QH / KH);
-    return AT_COUNTER_BYTES + sl_align_up(bh * S * G * AT_PART * sizeof(float), 256);
+    return AT_COUNTER_BYTES + sl_align_up(bh * AT_MAX_SPLITS * G * AT_PART * sizeof(float), 256);
 }
 
 int sl_attn_launch(attn_args a, void *ws, size_t ws_bytes, hipStream_t s) {
@@ -253,7 +264,9 @@ int sl_attn_launch(attn_args a, void *ws, size_t ws_bytes, hipStream_t s) {
     a.counter = static_cast<uint32_t *>(ws);
     SL_REQUIRE(static_cast<size_t>(a.B) * a.KH * sizeof(uint32_t) <= AT_COUNTER_BYTES, SL_ERR_UNSUPPORTED);
     a.part = reinterpret_cast<float *>(static_cast<char *>(ws) + AT_COUNTER_BYTES);
-    if (a.rows == 0) a.rows = pick_rows(a.B, a.KH, a.k);
+    if (a.rows <= 0) a.rows = pick_rows(a.B, a.KH, a.k);
+    SL_REQUIRE(a.rows % AT_ITER_ROWS == 0 && a.rows <= AT_MAX_ROWS, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE((a.k + a.rows - 1) / a.rows <= AT_MAX_SPLITS, SL_ERR_UNSUPPORTED);  // k <= 16384
     if (a.scale <= 0.f) a.scale = 0.08838834764831845f;  // 1/sqrt(128)
     switch (a.dtype) {
         case SL_F32: return dispatch_g<float>(a, s);

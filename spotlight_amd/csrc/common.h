@@ -151,6 +151,38 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// ---- cross-workgroup hand-off without cache-wide maintenance ----------------------
+// A partial result that another workgroup (possibly on another XCD, behind
+// another L2) will read is written and read with agent-scope relaxed atomics:
+// those accesses are coherent at device level by themselves, so no L2
+// write-back / invalidate of the whole cache is needed.  The writer then only
+// has to wait until its stores are acknowledged (publish_wait) before the
+// barrier that precedes the arrival ticket; a device-scope __threadfence()
+// instead costs a full L2 write-back and invalidate per wave.
+__device__ __forceinline__ void st_agent(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_agent(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(uint32_t *p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t ld_agent(const uint32_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// all earlier memory operations of this lane have completed
+__device__ __forceinline__ void publish_wait() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+}
+// Takes an arrival ticket for `counter`; true for the workgroup that arrives
+// last of `expected`.  Call after publish_wait() + __syncthreads(), from one lane.
+__device__ __forceinline__ bool arrive_last(uint32_t *counter, uint32_t expected) {
+    const uint32_t ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return ticket == expected - 1;
+}
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 

@@ -1,9 +1,11 @@
 // Fused decode step and the small library-level entry points.
 //
 // sl_decode_step enqueues, on one stream and without host synchronisation:
-//   1. hash_kernel       q codes -> workspace; new key's code, K and V -> cache row seq_lens[b]
+//   1. hash_kernel       q codes -> workspace; new key's code, K and V -> cache row seq_lens[b];
+//                        clears the score histogram
 //   2. hamming_kernel    fused flavour: head-major scores + global histogram over seq_lens[b]+1 rows
-//   3. select_kernel     threshold from the histogram, stable compaction -> idx
+//   3. select_fused_kernel (or select_count_kernel + select_compact_kernel beyond 64k rows)
+//                        threshold from the histogram, stable compaction -> idx
 //   4. lru_kernel        (optional) resident-table update -> slot list
 //   5. sparse_attn_kernel over idx (or over the resident slots), then seq_lens[b] += 1
 // Every length is read from device memory, so the same captured HIP graph can
@@ -24,7 +26,7 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, ui
 }
 
 struct ws_layout {
-    size_t q_code, hist, score, hash, attn, total;
+    size_t q_code, select, score, attn, total;
 };
 
 ws_layout layout(const sl_decode_params &p) {
@@ -33,9 +35,8 @@ ws_layout layout(const sl_decode_params &p) {
     const size_t G = static_cast<size_t>(p.QH / p.KH);
     size_t off = 0;
     L.q_code = off; off += sl_align_up(sizeof(uint32_t) * p.B * p.QH * W, 256);
-    L.hist = off;   off += sl_align_up(sizeof(uint32_t) * p.B * p.KH * (G * p.nbits + 1), 256);
+    L.select = off; off += sl_select_ws_bytes(p.B, p.KH, static_cast<int>(G * p.nbits + 1), p.n_cap);
     L.score = off;  off += sl_align_up(sizeof(int16_t) * p.B * p.KH * static_cast<size_t>(p.n_cap), 256);
-    L.hash = off;   off += sl_hash_ws_bytes(p.B, p.QH + p.KH, p.d_hid, p.nbits);
     L.attn = off;   off += sl_attn_ws_bytes(p.B, p.QH, p.KH, p.k);
     L.total = off;
     return L;
@@ -107,7 +108,6 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     char *ws = static_cast<char *>(p.ws);
     const int W = p.nbits / 32, G = p.QH / p.KH;
     uint32_t *q_code = reinterpret_cast<uint32_t *>(ws + L.q_code);
-    uint32_t *hist = reinterpret_cast<uint32_t *>(ws + L.hist);
     int16_t *score = reinterpret_cast<int16_t *>(ws + L.score);
 
     // 1. hash q and the new key; append code, K, V
@@ -128,14 +128,19 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     sk.copy_src[0] = p.k_new; sk.copy_dst[0] = p.keys;
     sk.copy_src[1] = p.v_new; sk.copy_dst[1] = p.vals;
     sk.copy_dst_stride_b = p.n_cap * p.KH * p.d; sk.copy_dst_stride_n = static_cast<int64_t>(p.KH) * p.d;
+    select_args ta{};
+    ta.B = p.B; ta.KH = p.KH; ta.n_bins = G * p.nbits + 1;
+    sl_select_carve(ta, ws + L.select, p.n_cap);
+    ha.zero_words = ta.hist;  // the scorer of this step starts from a clean histogram
+    ha.zero_count = static_cast<int64_t>(p.B) * p.KH * ta.n_bins * ta.hist_groups;
     if (stages & SL_STAGE_HASH) {
-        rc = sl_hash_launch(ha, ws + L.hash, L.attn - L.hash, s);
+        rc = sl_hash_launch(ha, s);
         if (rc != SL_OK) return rc;
     }
 
     // 2. score seq_lens[b] + 1 rows
     hamming_args sa{};
-    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = hist; sa.seq_lens = p.seq_lens;
+    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.seq_lens = p.seq_lens;
     sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
     sa.n_bins = G * p.nbits + 1; sa.len_bias = 1; sa.n = p.n_max; sa.n_cap = p.n_cap;
     sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
@@ -145,9 +150,8 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     }
 
     // 3. select
-    select_args ta{};
-    ta.score = score; ta.hist = hist; ta.idx = p.idx; ta.seq_lens = p.seq_lens;
-    ta.B = p.B; ta.KH = p.KH; ta.k = p.k; ta.n_bins = sa.n_bins; ta.len_bias = 1; ta.n = p.n_max;
+    ta.score = score; ta.idx = p.idx; ta.seq_lens = p.seq_lens;
+    ta.k = p.k; ta.len_bias = 1; ta.n = p.n_max;
     ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
     if (stages & SL_STAGE_SELECT) {
         rc = sl_select_launch(ta, s);

@@ -10,7 +10,8 @@ struct hamming_args {
     const uint32_t *q_code;   // [B, QH, W], batch stride q_stride_b words
     const uint32_t *k_code;   // [B, n, KH, W], batch stride k_stride_b words
     int16_t *out;             // plain: [B, n, KH]; fused: [B, KH, n_cap]
-    uint32_t *hist;           // fused: [B, KH, n_bins] global histogram
+    uint32_t *hist;           // fused: [B, KH, hist_groups, n_bins] global histogram copies
+    int hist_groups;
     const int32_t *seq_lens;  // optional per-batch token count
     int B, KH, G, W, head_map;
     int n_bins;               // fused: G*W*32 + 1

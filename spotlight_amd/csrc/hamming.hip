@@ -9,8 +9,8 @@
 // record and keeps that head's G query codes in registers.
 //
 // The fused flavour additionally (1) counts every score into an LDS histogram
-// [KH][G*nbits+1] and flushes the non-empty bins to the global histogram the
-// count-select kernel reads, and (2) writes the scores head-major
+// [KH][G*nbits+1] and flushes the non-empty bins to one of a few copies of the
+// global histogram the count-select kernel sums and reads, and (2) writes the scores head-major
 // [B, KH, n_cap] through an LDS transpose so that the selector streams one
 // contiguous int16 run per (b, kv head).
 #include "hamming.h"
@@ -82,18 +82,16 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     if constexpr (FUSED || G_T == 0) __syncthreads();
 
     const uint32_t *kb = a.k_code + static_cast<int64_t>(b) * a.k_stride_b;
+    // loads are unconditional (rows past the end re-read the last row and are
+    // discarded below): no branch sits between the HS_U loads
     uint32_t kreg[HS_U][W];
     bool valid[HS_U];
 #pragma unroll
     for (int u = 0; u < HS_U; ++u) {
         const int64_t t = t0 + static_cast<int64_t>(u) * tok_per_pass + tl;
         valid[u] = t < n_b;
-        if (valid[u]) {
-            load_code<W>(kb + (t * KH + h) * W, kreg[u]);
-        } else {
-#pragma unroll
-            for (int w = 0; w < W; ++w) kreg[u][w] = 0;
-        }
+        const int64_t tc = valid[u] ? t : n_b - 1;
+        load_code<W>(kb + (tc * KH + h) * W, kreg[u]);
     }
 
     const int full = G * W * 32;
@@ -135,10 +133,13 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
             int16_t *dst = a.out + (static_cast<int64_t>(b) * KH + hh) * a.n_cap + t;
             *reinterpret_cast<uint2 *>(dst) = v;
         }
-        uint32_t *gh = a.hist + static_cast<int64_t>(b) * KH * NB;
+        // hist_groups copies of the global histogram spread the same-bin adds of the
+        // many workgroups of one (b, kv head) over as many addresses
+        const int grp = blockIdx.x % a.hist_groups;
         for (int i = tid; i < KH * NB; i += HS_THREADS) {
             const uint32_t c = hist[i];
-            if (c) atomicAdd(&gh[i], c);
+            const int hh = i / NB, bin = i % NB;
+            if (c) atomicAdd(&a.hist[((static_cast<int64_t>(b) * KH + hh) * a.hist_groups + grp) * NB + bin], c);
         }
     }
 }

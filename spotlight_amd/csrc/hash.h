@@ -22,10 +22,8 @@ struct hash_args {
     hash_side side[2];
     int n_sides;
     int dtype, n_layers, B, d_in, d_hid, nbits, residue;
-    float *part;        // workspace [B][Htot][SPL][nbits]
-    float *hid;         // workspace [B][Htot][d_hid] (two layers + residue only)
-    uint32_t *counter;  // workspace [Htot]
+    uint32_t *zero_words;  // optional: words the launch also clears (next step's histogram)
+    int64_t zero_count;
 };
 
-size_t sl_hash_ws_bytes(int B, int Htot, int d_hid, int nbits);
-int sl_hash_launch(hash_args a, void *ws, size_t ws_bytes, hipStream_t s);
+int sl_hash_launch(hash_args a, hipStream_t s);

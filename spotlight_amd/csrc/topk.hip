@@ -4,24 +4,41 @@
 // a histogram instead of a sort:
 //   1. histogram of the scores (built by the fused scorer, or by
 //      score_hist_kernel for scores that come from elsewhere);
-//   2. one workgroup per (b, kv head) walks the bins from the best score down
-//      with a block prefix sum and finds the threshold bin `thr`, the number of
-//      tokens strictly above it, and how many tokens `need` of the threshold
-//      bin itself still fit;
-//   3. the same workgroup streams its scores in token order; lane-contiguous
-//      runs of 8 tokens plus a block prefix sum over packed (above, equal)
-//      counts give every kept token its output position
+//   2. walking the bins from the best score down with a block prefix sum gives
+//      the threshold bin `thr`, the number of tokens strictly above it, and how
+//      many tokens `need` of the threshold bin itself still fit;
+//   3. the scores are swept in token order; lane-contiguous runs of 8 tokens
+//      plus prefix sums over packed (above, equal) counts give every kept
+//      token its output position
 //          pos = #above before it + min(#equal before it, need),
 //      so the k kept tokens come out in ascending token order and ties at the
-//      threshold resolve to the lowest token index.  No sort, no atomics, and
-//      the result is the same on every run.
+//      threshold resolve to the lowest token index.  No sort, no atomics in
+//      the selection, and the result is the same on every run.
+//
+// Work is cut into blocks of 2048 tokens, one workgroup per (block, b, kv
+// head): a compute unit needs some 20 instructions per token, so one
+// workgroup per (b, kv head) would spend microseconds per 10k tokens.  Every
+// workgroup derives (thr, need) itself (the histogram is 2 KB).  What it also
+// needs is the number of tokens above / at the threshold in the blocks before
+// its own:
+//   * up to TK_FUSE_BLOCKS blocks, it simply counts them itself -- all those
+//     score loads are issued together with its own, one memory round trip,
+//     one launch (select_fused_kernel);
+//   * beyond that, a first launch writes per-block counts and a second one
+//     sums them (select_count_kernel + select_compact_kernel).
 #include "topk.h"
 
 namespace {
 
-constexpr int TK_CHUNKS = 4;             // 8-token runs per lane per pass
-constexpr int TK_RUN = 8;
-constexpr int TK_PASS_TOKENS = TK_THREADS * TK_RUN;  // tokens per chunk (8192)
+constexpr int TK_RUN = 8;                          // consecutive tokens per lane (one 16-byte load)
+constexpr int TK_BLOCK = TK_THREADS * TK_RUN;      // tokens per workgroup
+constexpr int TK_MAX_BPT = (TK_MAX_BINS + TK_THREADS - 1) / TK_THREADS;  // histogram bins a lane owns
+constexpr int TK_FUSE_BLOCKS = 32;                 // single-launch path up to this many blocks
+
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *p, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
 
 // ---- histogram of externally produced scores -------------------------------
 // One workgroup per (token block, b, group of heads whose bins fit 64 KiB of
@@ -29,17 +46,22 @@ constexpr int TK_PASS_TOKENS = TK_THREADS * TK_RUN;  // tokens per chunk (8192)
 constexpr int SH_THREADS = 256;
 constexpr int SH_TOKENS = 512;  // tokens per workgroup
 
+__device__ __forceinline__ int64_t tokens_of(const select_args &a, int b) {
+    int64_t n_b = a.n;
+    if (a.seq_lens) {
+        const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
+        n_b = l < n_b ? l : n_b;
+    }
+    return n_b;
+}
+
 __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, int heads_per_group) {
     extern __shared__ uint32_t hist[];
     const int b = blockIdx.y;
     const int NB = a.n_bins;
     const int h0 = blockIdx.z * heads_per_group;
     const int KHg = a.KH - h0 < heads_per_group ? a.KH - h0 : heads_per_group;  // heads of this group
-    int64_t n_b = a.n;
-    if (a.seq_lens) {
-        const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
-        n_b = l < n_b ? l : n_b;
-    }
+    const int64_t n_b = tokens_of(a, b);
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * SH_TOKENS;
     if (t0 >= n_b) return;
     for (int e = threadIdx.x; e < KHg * NB; e += SH_THREADS) hist[e] = 0;
@@ -56,156 +78,341 @@ __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, i
         atomicAdd(&hist[h * NB + s], 1u);
     }
     __syncthreads();
-    uint32_t *gh = a.hist + (static_cast<int64_t>(b) * a.KH + h0) * NB;
+    const int grp = blockIdx.x % a.hist_groups;
     for (int i = threadIdx.x; i < KHg * NB; i += SH_THREADS) {
         const uint32_t c = hist[i];
-        if (c) atomicAdd(&gh[i], c);
+        const int h = i / NB, bin = i % NB;
+        if (c) atomicAdd(&a.hist[((static_cast<int64_t>(b) * a.KH + h0 + h) * a.hist_groups + grp) * NB + bin], c);
     }
 }
 
-// ---- select -------------------------------------------------------------------
+// ---- pieces shared by the select kernels ---------------------------------------
 
+// Eight consecutive scores of one lane as four packed words (token 2j in the low
+// half of word j).  The load is unconditional and branch free: CONTIG reads the
+// 16 bytes at t0 (callers guarantee they lie inside the allocation), the strided
+// flavour clamps each token index; tokens at or beyond n_b then become -1, which
+// never qualifies.
 template <bool CONTIG>
-__global__ __launch_bounds__(TK_THREADS) void select_kernel(select_args a) {
-    __shared__ uint32_t s_wave[TK_CHUNKS][TK_THREADS / 64 + 1];
-    __shared__ int s_thr, s_need;
-
-    const int tid = threadIdx.x;
-    const int b = blockIdx.x / a.KH, h = blockIdx.x % a.KH;
-    const int NB = a.n_bins;
-    int64_t n_b = a.n;
-    if (a.seq_lens) {
-        const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
-        n_b = l < n_b ? l : n_b;
+__device__ __forceinline__ uint4 load_run(const select_args &a, const int16_t *sc, int64_t t0, int64_t n_b) {
+    uint32_t w[4];
+    if constexpr (CONTIG) {
+        const uint4 r = *reinterpret_cast<const uint4 *>(sc + t0);
+        w[0] = r.x; w[1] = r.y; w[2] = r.z; w[3] = r.w;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t t = t0 + 2 * j;
+            const int64_t last = n_b > 0 ? n_b - 1 : 0;
+            const uint32_t lo = static_cast<uint16_t>(sc[(t < last ? t : last) * a.stride_n]);
+            const uint32_t hi = static_cast<uint16_t>(sc[(t + 1 < last ? t + 1 : last) * a.stride_n]);
+            w[j] = lo | (hi << 16);
+        }
     }
-    const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int64_t t = t0 + 2 * j;
+        if (t >= n_b) w[j] |= 0xffffu;
+        if (t + 1 >= n_b) w[j] |= 0xffff0000u;
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
 
-    // -- threshold: lane `tid` owns bins NB-1 - (tid*BPT + j), best scores first
-    uint32_t *gh = a.hist + (static_cast<int64_t>(b) * a.KH + h) * NB;
+__device__ __forceinline__ void unpack_run(const uint4 &r, int (&v)[TK_RUN]) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        v[2 * j] = static_cast<int16_t>(w[j] & 0xffffu);
+        v[2 * j + 1] = static_cast<int16_t>(w[j] >> 16);
+    }
+}
+
+// Lane `tid` owns bins NB-1 - (tid*BPT + j), best scores first, and sums their NG
+// copies; every load of the lane is independent of the others (one round trip).
+template <int MAX_BPT, int NG>
+__device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, uint32_t (&cnt)[MAX_BPT]) {
+    const int NB = a.n_bins, tid = threadIdx.x;
     const int BPT = (NB + TK_THREADS - 1) / TK_THREADS;
-    uint32_t cnt[TK_MAX_BINS / TK_THREADS + 1];
+    const uint32_t *gh = a.hist + static_cast<int64_t>(bh) * NG * NB;
+    uint32_t raw[MAX_BPT][NG];
+#pragma unroll
+    for (int j = 0; j < MAX_BPT; ++j) {
+        const int bi = tid * BPT + j;
+        const bool live = j < BPT && bi < NB;
+        const int bin = live ? NB - 1 - bi : 0;  // unconditional loads, dead bins are dropped below
+#pragma unroll
+        for (int g = 0; g < NG; ++g) raw[j][g] = gh[g * NB + bin];
+    }
     uint32_t mine = 0;
 #pragma unroll
-    for (int j = 0; j < TK_MAX_BINS / TK_THREADS + 1; ++j) {
+    for (int j = 0; j < MAX_BPT; ++j) {
         const int bi = tid * BPT + j;
-        cnt[j] = 0;
-        if (j < BPT && bi < NB) {
-            cnt[j] = gh[NB - 1 - bi];
-            gh[NB - 1 - bi] = 0;  // leave the histogram ready for the next step
-        }
+        uint32_t c = 0;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) c += raw[j][g];
+        cnt[j] = (j < BPT && bi < NB) ? c : 0u;
         mine += cnt[j];
     }
-    if (tid == 0) { s_thr = NB; s_need = 0; }  // selects nothing unless a lane finds the bin
+    return mine;
+}
+
+// Block-wide search of the threshold bin; every lane returns (thr, need).
+template <int MAX_BPT>
+__device__ __forceinline__ void find_threshold(const select_args &a, const uint32_t (&cnt)[MAX_BPT],
+                                               uint32_t mine, int k_eff, uint32_t *s_wave, int *s_tn,
+                                               int &thr, int &need) {
+    const int NB = a.n_bins, tid = threadIdx.x;
+    const int BPT = (NB + TK_THREADS - 1) / TK_THREADS;
+    if (tid == 0) { s_tn[0] = NB; s_tn[1] = 0; }  // selects nothing unless a lane finds the bin
     uint32_t total;
-    uint32_t cum = block_exclusive_sum<TK_THREADS>(mine, s_wave[0], &total);
+    uint32_t cum = block_exclusive_sum<TK_THREADS>(mine, s_wave, &total);
 #pragma unroll
-    for (int j = 0; j < TK_MAX_BINS / TK_THREADS + 1; ++j) {
+    for (int j = 0; j < MAX_BPT; ++j) {
         if (k_eff > 0 && cum < static_cast<uint32_t>(k_eff) && cum + cnt[j] >= static_cast<uint32_t>(k_eff)) {
-            s_thr = NB - 1 - (tid * BPT + j);
-            s_need = k_eff - static_cast<int>(cum);
+            s_tn[0] = NB - 1 - (tid * BPT + j);
+            s_tn[1] = k_eff - static_cast<int>(cum);
         }
         cum += cnt[j];
     }
     __syncthreads();
-    const int thr = s_thr, need = s_need;
+    thr = s_tn[0];
+    need = s_tn[1];
+}
 
-    // -- compaction in token order
-    int32_t *out = a.idx + (static_cast<int64_t>(b) * a.KH + h) * a.k;
-    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
-    uint32_t run_gt = 0, run_eq = 0;  // kept-above / equal tokens seen in earlier passes
-
-    for (int64_t base = 0; base < n_b; base += static_cast<int64_t>(TK_PASS_TOKENS) * TK_CHUNKS) {
-        int16_t v[TK_CHUNKS][TK_RUN];
-        uint32_t packed[TK_CHUNKS];
+__device__ __forceinline__ uint32_t count_run(const uint4 &r, int thr) {
+    int v[TK_RUN];
+    unpack_run(r, v);
+    uint32_t gt = 0, eq = 0;
 #pragma unroll
-        for (int c = 0; c < TK_CHUNKS; ++c) {
-            const int64_t t0 = base + static_cast<int64_t>(c) * TK_PASS_TOKENS + tid * TK_RUN;
-            if (CONTIG && t0 + TK_RUN <= n_b) {
-                const uint4 w = *reinterpret_cast<const uint4 *>(sc + t0);
-                const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    v[c][2 * j] = static_cast<int16_t>(ws[j] & 0xffffu);
-                    v[c][2 * j + 1] = static_cast<int16_t>(ws[j] >> 16);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < TK_RUN; ++j)
-                    v[c][j] = (t0 + j < n_b) ? sc[(t0 + j) * a.stride_n] : static_cast<int16_t>(-1);
-            }
-            uint32_t gt = 0, eq = 0;
-#pragma unroll
-            for (int j = 0; j < TK_RUN; ++j) {
-                gt += v[c][j] > thr;
-                eq += v[c][j] == thr;
-            }
-            packed[c] = gt | (eq << 16);
-        }
-        // TK_CHUNKS block scans sharing two barriers
-        uint32_t inc[TK_CHUNKS];
-#pragma unroll
-        for (int c = 0; c < TK_CHUNKS; ++c) {
-            inc[c] = wave_inclusive_sum(packed[c]);
-            if (lane_id() == 63) s_wave[c][wave_id()] = inc[c];
-        }
-        __syncthreads();
-        if (tid < 64 * TK_CHUNKS) {
-            const int c = tid >> 6, l = tid & 63;
-            const uint32_t t = l < TK_THREADS / 64 ? s_wave[c][l] : 0u;
-            const uint32_t ti = wave_inclusive_sum(t);
-            if (l < TK_THREADS / 64) s_wave[c][l] = ti - t;
-            if (l == 63) s_wave[c][TK_THREADS / 64] = ti;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int c = 0; c < TK_CHUNKS; ++c) {
-            const uint32_t ex = s_wave[c][wave_id()] + inc[c] - packed[c];
-            uint32_t gt_before = run_gt + (ex & 0xffffu);
-            uint32_t eq_before = run_eq + (ex >> 16);
-            const int64_t t0 = base + static_cast<int64_t>(c) * TK_PASS_TOKENS + tid * TK_RUN;
-#pragma unroll
-            for (int j = 0; j < TK_RUN; ++j) {
-                const int s = v[c][j];
-                if (s > thr) {
-                    const uint32_t pos = gt_before + (eq_before < static_cast<uint32_t>(need) ? eq_before : static_cast<uint32_t>(need));
-                    if (pos < static_cast<uint32_t>(k_eff)) out[pos] = static_cast<int32_t>(t0 + j);
-                    ++gt_before;
-                } else if (s == thr) {
-                    if (eq_before < static_cast<uint32_t>(need)) {
-                        const uint32_t pos = gt_before + eq_before;
-                        if (pos < static_cast<uint32_t>(k_eff)) out[pos] = static_cast<int32_t>(t0 + j);
-                    }
-                    ++eq_before;
-                }
-            }
-            const uint32_t tot = s_wave[c][TK_THREADS / 64];
-            run_gt += tot & 0xffffu;
-            run_eq += tot >> 16;
-        }
-        __syncthreads();  // s_wave is rewritten by the next pass
-        const uint32_t kept = run_gt + (run_eq < static_cast<uint32_t>(need) ? run_eq : static_cast<uint32_t>(need));
-        if (kept >= static_cast<uint32_t>(k_eff)) break;
+    for (int j = 0; j < TK_RUN; ++j) {
+        gt += v[j] > thr;
+        eq += v[j] == thr;
     }
-    for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;
+    return gt | (eq << 16);
+}
+
+// Places the kept tokens of one block.  (tg, te): tokens above / at the threshold
+// in all earlier blocks.  Contains barriers.
+__device__ __forceinline__ void place_block(const uint4 &run, int64_t t0, int thr, int need, int k_eff,
+                                            uint32_t tg, uint32_t te, uint32_t *s_wave, int32_t *out) {
+    const uint32_t uneed = static_cast<uint32_t>(need);
+    uint32_t tot;
+    const uint32_t ex = block_exclusive_sum<TK_THREADS>(count_run(run, thr), s_wave, &tot);
+    int v[TK_RUN];
+    unpack_run(run, v);
+    uint32_t gt_before = tg + (ex & 0xffffu), eq_before = te + (ex >> 16);
+#pragma unroll
+    for (int j = 0; j < TK_RUN; ++j) {
+        const int s = v[j];
+        if (s > thr) {
+            const uint32_t pos = gt_before + (eq_before < uneed ? eq_before : uneed);
+            if (pos < static_cast<uint32_t>(k_eff)) out[pos] = static_cast<int32_t>(t0 + j);
+            ++gt_before;
+        } else if (s == thr) {
+            if (eq_before < uneed) {
+                const uint32_t pos = gt_before + eq_before;
+                if (pos < static_cast<uint32_t>(k_eff)) out[pos] = static_cast<int32_t>(t0 + j);
+            }
+            ++eq_before;
+        }
+    }
+}
+
+// ---- single launch: every block counts the blocks before it ---------------------
+
+// Body for a block with at most NPREV blocks before it: the NPREV loads are
+// unconditional (slots beyond `blk` re-read the own block and are not counted).
+template <bool CONTIG, int MAX_BPT, int NG, int NPREV>
+__device__ __forceinline__ void select_fused_body(const select_args &a, int blk, int bh, int b, int h, int64_t n_b,
+                                                  int k_eff, int32_t *out, uint32_t *s_wave, int *s_tn) {
+    const int tid = threadIdx.x;
+    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
+    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
+    const uint4 v = load_run<CONTIG>(a, sc, t0, n_b);
+    uint4 prev[NPREV > 0 ? NPREV : 1];
+#pragma unroll
+    for (int j = 0; j < NPREV; ++j)
+        prev[j] = load_run<CONTIG>(a, sc, static_cast<int64_t>(j < blk ? j : blk) * TK_BLOCK + tid * TK_RUN, n_b);
+    uint32_t cnt[MAX_BPT];
+    const uint32_t mine = load_bins<MAX_BPT, NG>(a, bh, cnt);
+
+    int thr, need;
+    find_threshold<MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+
+    uint32_t pg = 0, pe = 0;
+#pragma unroll
+    for (int j = 0; j < NPREV; ++j) {
+        const uint32_t c = j < blk ? count_run(prev[j], thr) : 0u;
+        pg += c & 0xffffu;
+        pe += c >> 16;
+    }
+    uint32_t tg, te;
+    block_exclusive_sum<TK_THREADS>(pg, s_wave, &tg);
+    __syncthreads();
+    block_exclusive_sum<TK_THREADS>(pe, s_wave, &te);
+    __syncthreads();
+    const uint32_t uneed = static_cast<uint32_t>(need);
+    if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
+    place_block(v, t0, thr, need, k_eff, tg, te, s_wave, out);
+}
+
+template <bool CONTIG, int MAX_BPT, int NG>
+__global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a) {
+    __shared__ uint32_t s_wave[TK_THREADS / 64 + 1];
+    __shared__ int s_tn[2];
+    const int tid = threadIdx.x;
+    const int blk = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / a.KH, h = bh % a.KH;
+    const int64_t n_b = tokens_of(a, b);
+    const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
+    int32_t *out = a.idx + static_cast<int64_t>(bh) * a.k;
+    if (blk == 0)
+        for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;
+    if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b) return;
+    if (blk == 0) select_fused_body<CONTIG, MAX_BPT, NG, 0>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
+    else if (blk <= 3) select_fused_body<CONTIG, MAX_BPT, NG, 3>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
+    else if (blk <= 7) select_fused_body<CONTIG, MAX_BPT, NG, 7>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
+    else if (blk <= 15) select_fused_body<CONTIG, MAX_BPT, NG, 15>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
+    else select_fused_body<CONTIG, MAX_BPT, NG, TK_FUSE_BLOCKS - 1>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
+}
+
+// ---- two launches: per-block counts, then placement --------------------------------
+
+template <bool CONTIG, int MAX_BPT, int NG>
+__global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a) {
+    __shared__ uint32_t s_wave[TK_THREADS / 64 + 1];
+    __shared__ int s_tn[2];
+    const int tid = threadIdx.x;
+    const int blk = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / a.KH, h = bh % a.KH;
+    const int64_t n_b = tokens_of(a, b);
+    if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b && blk > 0) return;
+    const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
+
+    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
+    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
+    const uint4 v = load_run<CONTIG>(a, sc, t0, n_b);
+    uint32_t cnt[MAX_BPT];
+    const uint32_t mine = load_bins<MAX_BPT, NG>(a, bh, cnt);
+    int thr, need;
+    find_threshold<MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+    if (blk == 0 && tid == 0) {
+        a.thr_need[bh * 2] = thr;
+        a.thr_need[bh * 2 + 1] = need;
+    }
+    uint32_t tot;
+    block_exclusive_sum<TK_THREADS>(count_run(v, thr), s_wave, &tot);
+    if (tid == 0) a.block_cnt[static_cast<int64_t>(bh) * a.n_blocks + blk] = tot;
+}
+
+template <bool CONTIG>
+__global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args a) {
+    __shared__ uint32_t s_wave[TK_THREADS / 64 + 1];
+    const int tid = threadIdx.x;
+    const int blk = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / a.KH, h = bh % a.KH;
+    const int64_t n_b = tokens_of(a, b);
+    const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
+    int32_t *out = a.idx + static_cast<int64_t>(bh) * a.k;
+    if (blk == 0)
+        for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;
+    if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b) return;
+    const int thr = a.thr_need[bh * 2], need = a.thr_need[bh * 2 + 1];
+
+    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
+    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
+    const uint4 v = load_run<CONTIG>(a, sc, t0, n_b);
+
+    const uint32_t *bc = a.block_cnt + static_cast<int64_t>(bh) * a.n_blocks;
+    uint32_t pg = 0, pe = 0;
+    for (int j = tid; j < blk; j += TK_THREADS) {
+        const uint32_t c = bc[j];
+        pg += c & 0xffffu;
+        pe += c >> 16;
+    }
+    uint32_t tg, te;
+    block_exclusive_sum<TK_THREADS>(pg, s_wave, &tg);
+    __syncthreads();
+    block_exclusive_sum<TK_THREADS>(pe, s_wave, &te);
+    __syncthreads();
+    const uint32_t uneed = static_cast<uint32_t>(need);
+    if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
+    place_block(v, t0, thr, need, k_eff, tg, te, s_wave, out);
 }
 
 }  // namespace
 
+int sl_select_hist_groups(int64_t n) {
+    // Copies of every histogram bin, so that the same-bin adds of the many scorer
+    // workgroups of one (b, kv head) spread over as many addresses: 16 for long
+    // caches, 4 for short ones (fewer workgroups, and the copies must be cleared
+    // and read every step).
+    return n > 20000 ? 16 : 4;
+}
+
+size_t sl_select_ws_bytes(int B, int KH, int n_bins, int64_t n) {
+    const size_t bh = static_cast<size_t>(B) * KH;
+    const size_t n_blocks = static_cast<size_t>((n + TK_BLOCK - 1) / TK_BLOCK);
+    return sl_align_up(sizeof(uint32_t) * bh * n_bins * sl_select_hist_groups(n), 256) +
+           sl_align_up(sizeof(int32_t) * bh * 2, 256) +
+           sl_align_up(sizeof(uint32_t) * bh * (n_blocks ? n_blocks : 1), 256);
+}
+
+void sl_select_carve(select_args &a, void *ws, int64_t n_for_blocks) {
+    const size_t bh = static_cast<size_t>(a.B) * a.KH;
+    char *p = static_cast<char *>(ws);
+    a.hist = reinterpret_cast<uint32_t *>(p);
+    a.hist_groups = sl_select_hist_groups(n_for_blocks);
+    p += sl_align_up(sizeof(uint32_t) * bh * a.n_bins * a.hist_groups, 256);
+    a.thr_need = reinterpret_cast<int32_t *>(p);
+    p += sl_align_up(sizeof(int32_t) * bh * 2, 256);
+    a.block_cnt = reinterpret_cast<uint32_t *>(p);
+    a.n_blocks = static_cast<int>((n_for_blocks + TK_BLOCK - 1) / TK_BLOCK);
+    if (a.n_blocks < 1) a.n_blocks = 1;
+}
+
 int sl_select_launch(const select_args &a, hipStream_t s) {
-    const int64_t blocks = static_cast<int64_t>(a.B) * a.KH;
-    SL_REQUIRE(blocks <= 0x7fffffffLL, SL_ERR_UNSUPPORTED);
+    const int64_t bh = static_cast<int64_t>(a.B) * a.KH;
+    SL_REQUIRE(bh <= 65535, SL_ERR_UNSUPPORTED);
     SL_REQUIRE(a.n_bins >= 1 && a.n_bins <= TK_MAX_BINS, SL_ERR_UNSUPPORTED);
-    const bool contig = a.stride_n == 1 && sl_aligned(a.score, 16) && a.stride_b % 8 == 0 && a.stride_h % 8 == 0;
-    if (contig)
-        select_kernel<true><<<dim3(static_cast<unsigned>(blocks)), dim3(TK_THREADS), 0, s>>>(a);
-    else
-        select_kernel<false><<<dim3(static_cast<unsigned>(blocks)), dim3(TK_THREADS), 0, s>>>(a);
+    int64_t blocks = (a.n + TK_BLOCK - 1) / TK_BLOCK;
+    if (blocks < 1) blocks = 1;
+    SL_REQUIRE(blocks <= a.n_blocks, SL_ERR_WORKSPACE);
+    // the 16-byte loads may run up to 7 tokens past a.n: allowed when rows are padded to 8 tokens
+    const bool contig = a.stride_n == 1 && sl_aligned(a.score, 16) && a.stride_b % 8 == 0 && a.stride_h % 8 == 0 &&
+                        a.stride_h >= (a.n + 7) / 8 * 8;
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(bh));
+    const bool small = a.n_bins <= 4 * TK_THREADS;  // few bins per lane: the common case
+    SL_REQUIRE(a.hist_groups == 4 || a.hist_groups == 16, SL_ERR_UNSUPPORTED);
+#define SL_SELECT_LAUNCH(CONTIG, BPT, NG)                                                        \
+    do {                                                                                         \
+        if (blocks <= TK_FUSE_BLOCKS) {                                                          \
+            select_fused_kernel<CONTIG, BPT, NG><<<grid, dim3(TK_THREADS), 0, s>>>(a);           \
+        } else {                                                                                 \
+            select_count_kernel<CONTIG, BPT, NG><<<grid, dim3(TK_THREADS), 0, s>>>(a);           \
+            select_compact_kernel<CONTIG><<<grid, dim3(TK_THREADS), 0, s>>>(a);                  \
+        }                                                                                        \
+    } while (0)
+#define SL_SELECT_NG(CONTIG, BPT)                                 \
+    do {                                                          \
+        if (a.hist_groups == 16) SL_SELECT_LAUNCH(CONTIG, BPT, 16); \
+        else SL_SELECT_LAUNCH(CONTIG, BPT, 4);                    \
+    } while (0)
+    if (contig) {
+        if (small) SL_SELECT_NG(true, 4);
+        else SL_SELECT_NG(true, TK_MAX_BPT);
+    } else {
+        if (small) SL_SELECT_NG(false, 4);
+        else SL_SELECT_NG(false, TK_MAX_BPT);
+    }
+#undef SL_SELECT_NG
+#undef SL_SELECT_LAUNCH
     return sl_check_launch();
 }
 
-extern "C" size_t sl_topk_workspace_bytes(int B, int KH, int max_score) {
-    if (B <= 0 || KH <= 0 || max_score < 0) return 0;
-    return sl_align_up(sizeof(uint32_t) * static_cast<size_t>(B) * KH * (static_cast<size_t>(max_score) + 1), 256);
+extern "C" size_t sl_topk_workspace_bytes(int B, int KH, int max_score, int64_t n) {
+    if (B <= 0 || KH <= 0 || max_score < 0 || n < 0) return 0;
+    return sl_select_ws_bytes(B, KH, max_score + 1, n);
 }
 
 extern "C" int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
@@ -216,18 +423,21 @@ extern "C" int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t st
     SL_REQUIRE(score && idx, SL_ERR_NULL);
     SL_REQUIRE(max_score + 1 <= TK_MAX_BINS, SL_ERR_UNSUPPORTED);
     SL_REQUIRE(n <= 0x7fffffffLL && B <= 65535, SL_ERR_UNSUPPORTED);
-    SL_REQUIRE(ws && ws_bytes >= sl_topk_workspace_bytes(B, KH, max_score), SL_ERR_WORKSPACE);
-    SL_REQUIRE(sl_aligned(ws, 4), SL_ERR_ALIGN);
+    SL_REQUIRE(ws && ws_bytes >= sl_topk_workspace_bytes(B, KH, max_score, n), SL_ERR_WORKSPACE);
+    SL_REQUIRE(sl_aligned(ws, 16), SL_ERR_ALIGN);
     const int n_bins = max_score + 1;
     int heads_per_group = 16384 / n_bins;  // 64 KiB of LDS bins per workgroup
     if (heads_per_group > KH) heads_per_group = KH;
     const int groups = (KH + heads_per_group - 1) / heads_per_group;
     const size_t lds = sizeof(uint32_t) * static_cast<size_t>(heads_per_group) * n_bins;
     select_args a{};
-    a.score = score; a.hist = static_cast<uint32_t *>(ws); a.idx = idx; a.seq_lens = seq_lens;
-    a.B = B; a.KH = KH; a.k = k; a.n_bins = max_score + 1; a.len_bias = 0; a.n = n;
+    a.score = score; a.idx = idx; a.seq_lens = seq_lens;
+    a.B = B; a.KH = KH; a.k = k; a.n_bins = n_bins; a.len_bias = 0; a.n = n;
     a.stride_b = stride_b; a.stride_n = stride_n; a.stride_h = stride_h;
+    sl_select_carve(a, ws, n);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t hist_words = static_cast<int64_t>(B) * KH * n_bins * a.hist_groups;
+    zero_words_kernel<<<dim3(static_cast<unsigned>((hist_words + 255) / 256)), dim3(256), 0, s>>>(a.hist, hist_words);
     if (n > 0) {
         const dim3 grid(static_cast<unsigned>((n + SH_TOKENS - 1) / SH_TOKENS), B, groups);
         score_hist_kernel<<<grid, dim3(SH_THREADS), lds, s>>>(a, heads_per_group);

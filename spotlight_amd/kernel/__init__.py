@@ -65,7 +65,9 @@ class Workspace:
 _default_ws = {}
 
 
-def _ws(kind: str, nbytes: int, device) -> torch.Tensor:
+def _ws(kind, nbytes: int, device) -> torch.Tensor:
+    """Default workspace of one op and one shape family on one device (parts of a
+    workspace must stay zero between calls, and where they lie depends on the shapes)."""
     key = (kind, torch.device(device))
     return _default_ws.setdefault(key, Workspace()).get(nbytes, device)
 
@@ -203,8 +205,8 @@ def topk_select(score: torch.Tensor, k: int, max_score: int,
         raise ValueError(layout)
     idx = torch.empty((B, KH, k), dtype=torch.int32, device=score.device)
     with torch.cuda.device(score.device):
-        nbytes = _L.sl_topk_workspace_bytes(B, KH, max_score)
-        ws = _ws("topk", nbytes, score.device)
+        nbytes = _L.sl_topk_workspace_bytes(B, KH, max_score, n)
+        ws = _ws(("topk", B, KH, max_score), nbytes, score.device)
         _lib.check(_L.sl_topk_select(
             score.data_ptr(), sb, sn, sh, idx.data_ptr(), B, n, KH, k, max_score,
             seq_lens.data_ptr() if seq_lens is not None else None, ws.data_ptr(), ws.numel(), _stream()),
@@ -285,12 +287,10 @@ def hash_mlp_pack(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor],
     codes = torch.empty((B, H, nbits // 32), dtype=torch.uint32, device=x.device)
     ptr = lambda t: t.data_ptr() if t is not None else None
     with torch.cuda.device(x.device):
-        nbytes = _L.sl_hash_workspace_bytes(B, H, d_hid, nbits)
-        ws = _ws("hash", nbytes, x.device)
         _lib.check(_L.sl_hash_mlp_pack(
             xc.data_ptr(), w1.data_ptr(), ptr(b1), ptr(w2), ptr(b2), codes.data_ptr(), _dtype(x), n_layers,
             B, H, d_in, d_hid, nbits, int(residue), xc.stride(0), codes.stride(0), codes.stride(1), 0, None,
-            ws.data_ptr(), ws.numel(), _stream()), "sl_hash_mlp_pack")
+            _stream()), "sl_hash_mlp_pack")
     return codes
 
 
