@@ -69,6 +69,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--layers", type=int, default=None)
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="launch heuristic passed to sl_tune (e.g. attn_target_wgs=128)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-breakdown", action="store_true")
     args = ap.parse_args()
@@ -81,6 +83,9 @@ def main():
 
     from spotlight_amd import _lib, decode, kernel
 
+    for kv in args.tune:
+        key, val = kv.split("=")
+        _lib.check(_lib.load().sl_tune(key.encode(), int(val)), f"sl_tune({kv})")
     c = dict(CONFIGS[args.config])
     L = args.layers or c["layers"]
     steps = args.steps if args.steps is not None else (256 if args.config == "c3" else 1000)

@@ -43,6 +43,11 @@ typedef enum { SL_HEADMAP_INTERLEAVED = 0, SL_HEADMAP_BLOCKED = 1 } sl_head_map;
 const char *sl_strerror(int status);
 int sl_version(void);
 
+/* Process-wide launch heuristics (host memory, not thread safe).  Keys:
+ * "attn_target_wgs": workgroups the attention launch aims for (default 256);
+ * it decides into how many runs the selected rows of a (b, kv head) are cut. */
+int sl_tune(const char *key, int value);
+
 /* ---- (a) sign -> packed codes ------------------------------------------ */
 
 /* Replaces packbits() (spotlight/kernel/packbits.cu:28-63) and

@@ -13,12 +13,15 @@
 //     registers and carries its own running softmax state (max, sum, 8
 //     accumulators per query head), so the G heads of the group reuse every
 //     K/V byte from registers and there is no barrier inside the row loop;
-//   * the 16 lane-group states are merged with shuffles and LDS; a run's
+//   * the 16 lane-group states meet in LDS: one weight exp(m - M) per (group,
+//     head), then every output element is a 16-term weighted sum; a run's
 //     (acc, max, sum) goes to the workspace through device-coherent stores;
 //     the last workgroup of a (b, kv head) to arrive loads all runs'
-//     partials at once (one round trip) and merges them in run order, so
-//     the result does not depend on arrival order.
+//     partials at once (one round trip) and merges them the same way, in run
+//     order, so the result does not depend on arrival order.
 #include "attn.h"
+
+#include <string.h>
 
 namespace {
 
@@ -37,8 +40,8 @@ constexpr size_t AT_COUNTER_BYTES = 64 * 1024;
 template <typename T, int G>
 __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
     __shared__ int s_row[AT_MAX_ROWS];
-    __shared__ float s_m[4][G], s_l[4][G];
-    __shared__ __align__(16) float s_acc[4][G][AT_D];
+    __shared__ float s_m[16][G], s_l[16][G], s_w[16][G], s_M[G], s_L[G];
+    __shared__ __align__(16) float s_acc[16][G][AT_D];  // 8 KB per query head of the group
     __shared__ int s_last;
 
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -123,28 +126,31 @@ __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
         }
     }
 
-    // merge the 4 lane groups of the wave, then the 4 waves
+    // every 16-lane group parks its state in LDS; the merge weights exp(m - M) are
+    // computed once per (group, head), then each output element sums 16 products
+    if (sub == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) { s_m[rslot][g] = m[g]; s_l[rslot][g] = l[g]; }
+    }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        float mw = fmaxf(m[g], __shfl_xor(m[g], 16, 64));
-        mw = fmaxf(mw, __shfl_xor(mw, 32, 64));
-        const float sc = mw == -INFINITY ? 0.f : __expf(m[g] - mw);
-        float lw = l[g] * sc;
-        lw += __shfl_xor(lw, 16, 64);
-        lw += __shfl_xor(lw, 32, 64);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            float v = acc[g][j] * sc;
-            v += __shfl_xor(v, 16, 64);
-            v += __shfl_xor(v, 32, 64);
-            acc[g][j] = v;
-        }
-        if (lane < 16) {
-            float4 *dst = reinterpret_cast<float4 *>(&s_acc[wave][g][sub * 8]);
-            dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
-            dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
-            if (sub == 0) { s_m[wave][g] = mw; s_l[wave][g] = lw; }
-        }
+        float4 *dst = reinterpret_cast<float4 *>(&s_acc[rslot][g][sub * 8]);
+        dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+        dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+    }
+    __syncthreads();
+    if (tid < G * 16) {  // lane (g, slot): weight of that slot, and the head's max / sum
+        const int g = tid >> 4, slot = tid & 15;
+        const float mine = s_m[slot][g];
+        float M = mine;
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_QUAD_XOR1>(0, __float_as_int(M))));
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_QUAD_XOR2>(0, __float_as_int(M))));
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_ROW_ROR4>(0, __float_as_int(M))));
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_ROW_ROR8>(0, __float_as_int(M))));
+        const float w = mine == -INFINITY ? 0.f : __expf(mine - M);
+        const float L = row16_sum(s_l[slot][g] * w);
+        s_w[slot][g] = w;
+        if (slot == 0) { s_M[g] = M; s_L[g] = L; }
     }
     __syncthreads();
 
@@ -153,22 +159,14 @@ __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
     float *part = a.part + (static_cast<int64_t>(bh) * S + split) * G * AT_PART;
     for (int e = tid; e < G * AT_D; e += AT_THREADS) {
         const int g = e / AT_D, c = e % AT_D;
-        float M = fmaxf(fmaxf(s_m[0][g], s_m[1][g]), fmaxf(s_m[2][g], s_m[3][g]));
-        float O = 0.f, L = 0.f;
+        float O = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float sc = M == -INFINITY ? 0.f : __expf(s_m[w][g] - M);
-            O = fmaf(s_acc[w][g][c], sc, O);
-            L = fmaf(s_l[w][g], sc, L);
-        }
+        for (int slot = 0; slot < 16; ++slot) O = fmaf(s_acc[slot][g][c], s_w[slot][g], O);
         if (S == 1) {
+            const float L = s_L[g];
             ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         } else {
             st_agent(part + g * AT_PART + c, O);
-            if (c == 0) {
-                st_agent(part + g * AT_PART + AT_D, M);
-                st_agent(part + g * AT_PART + AT_D + 1, L);
-            }
         }
     }
     if (S == 1) {
@@ -178,35 +176,66 @@ __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
         }
         return;
     }
+    if (tid < G) {
+        st_agent(part + tid * AT_PART + AT_D, s_M[tid]);
+        st_agent(part + tid * AT_PART + AT_D + 1, s_L[tid]);
+    }
     publish_wait();
     __syncthreads();
     if (tid == 0) s_last = arrive_last(&a.counter[bh], static_cast<uint32_t>(S));
     __syncthreads();
     if (!s_last) return;
 
-    // merge the S runs by log-sum-exp: every partial this lane needs is loaded at once
+    // merge the S runs by log-sum-exp.  All loads are issued together: the runs'
+    // accumulators by every lane, their (max, sum) by the first G*16 lanes, which
+    // turn them into one weight per (run, head) for everybody.
     const float *pb = a.part + static_cast<int64_t>(bh) * S * G * AT_PART;
-    for (int e = tid; e < G * AT_D; e += AT_THREADS) {
+    float pa[2][AT_MAX_SPLITS];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = tid + i * AT_THREADS;
         const int g = e / AT_D, c = e % AT_D;
-        float pm[AT_MAX_SPLITS], pl[AT_MAX_SPLITS], pa[AT_MAX_SPLITS];
 #pragma unroll
-        for (int s = 0; s < AT_MAX_SPLITS; ++s) {
-            const float *ps = pb + (static_cast<int64_t>(s) * G + g) * AT_PART;
-            pm[s] = s < S ? ld_agent(ps + AT_D) : -INFINITY;
-            pl[s] = s < S ? ld_agent(ps + AT_D + 1) : 0.f;
-            pa[s] = s < S ? ld_agent(ps + c) : 0.f;
+        for (int sp = 0; sp < AT_MAX_SPLITS; ++sp)
+            pa[i][sp] = (e < G * AT_D && sp < S) ? ld_agent(pb + (static_cast<int64_t>(sp) * G + g) * AT_PART + c) : 0.f;
+    }
+    if (tid < G * 16) {
+        const int g = tid >> 4, sp = tid & 15;
+        const float *ps = pb + (static_cast<int64_t>(sp < S ? sp : 0) * G + g) * AT_PART;
+        const float mine = sp < S ? ld_agent(ps + AT_D) : -INFINITY;
+        const float lmine = sp < S ? ld_agent(ps + AT_D + 1) : 0.f;
+        float M = mine;
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_QUAD_XOR1>(0, __float_as_int(M))));
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_QUAD_XOR2>(0, __float_as_int(M))));
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_ROW_ROR4>(0, __float_as_int(M))));
+        M = fmaxf(M, __int_as_float(dpp_i32<DPP_ROW_ROR8>(0, __float_as_int(M))));
+        const float w = mine == -INFINITY ? 0.f : __expf(mine - M);
+        const float L = row16_sum(lmine * w);
+        s_w[sp][g] = w;
+        if (sp == 0) s_L[g] = L;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int e = tid + i * AT_THREADS;
+        if (e < G * AT_D) {
+            const int g = e / AT_D;
+            float O = 0.f;
+#pragma unroll
+            for (int sp = 0; sp < AT_MAX_SPLITS; ++sp) O = fmaf(pa[i][sp], s_w[sp][g], O);
+            const float L = s_L[g];
+            ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         }
-        float M = -INFINITY;
-#pragma unroll
-        for (int s = 0; s < AT_MAX_SPLITS; ++s) M = fmaxf(M, pm[s]);
-        float L = 0.f, O = 0.f;
-#pragma unroll
-        for (int s = 0; s < AT_MAX_SPLITS; ++s) {
-            const float w = pm[s] == -INFINITY ? 0.f : __expf(pm[s] - M);
-            L = fmaf(pl[s], w, L);
-            O = fmaf(pa[s], w, O);
+    }
+    if (G * AT_D > 2 * AT_THREADS) {  // more than two outputs per lane (G > 4): the rest, plainly
+        for (int e = tid + 2 * AT_THREADS; e < G * AT_D; e += AT_THREADS) {
+            const int g = e / AT_D, c = e % AT_D;
+            float O = 0.f;
+            for (int sp = 0; sp < S; ++sp)
+                O = fmaf(ld_agent(pb + (static_cast<int64_t>(sp) * G + g) * AT_PART + c), s_w[sp][g], O);
+            const float L = s_L[g];
+            ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         }
-        ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
     }
     if (tid == 0) {
         st_agent(&a.counter[bh], 0u);
@@ -239,9 +268,11 @@ int dispatch_g(const attn_args &a, hipStream_t s) {
 
 // Rows per run: about one workgroup per compute unit over the whole launch,
 // never more than AT_MAX_SPLITS runs per (b, kv head), whole 64-row iterations.
+int g_attn_target_wgs = 256;  // sl_tune("attn_target_wgs", n)
+
 int pick_rows(int B, int KH, int k) {
     const int64_t bh = static_cast<int64_t>(B) * KH;
-    int64_t want = (256 + bh - 1) / bh;
+    int64_t want = (g_attn_target_wgs + bh - 1) / bh;
     if (want < 1) want = 1;
     if (want > AT_MAX_SPLITS) want = AT_MAX_SPLITS;
     int rows = static_cast<int>((k + want - 1) / want);
@@ -250,6 +281,11 @@ int pick_rows(int B, int KH, int k) {
 }
 
 }  // namespace
+
+int sl_attn_tune(const char *key, int value) {
+    if (!strcmp(key, "attn_target_wgs") && value > 0) { g_attn_target_wgs = value; return SL_OK; }
+    return SL_ERR_UNSUPPORTED;
+}
 
 size_t sl_attn_ws_bytes(int B, int QH, int KH, int k) {
     if (B <= 0 || QH <= 0 || KH <= 0 || k <= 0) return 0;

@@ -73,6 +73,11 @@ extern "C" const char *sl_strerror(int status) {
 
 extern "C" int sl_version(void) { return 100; }
 
+extern "C" int sl_tune(const char *key, int value) {
+    SL_REQUIRE(key, SL_ERR_NULL);
+    return sl_attn_tune(key, value);
+}
+
 extern "C" int sl_workspace_init(void *ws, size_t ws_bytes, void *stream) {
     if (ws_bytes == 0) return SL_OK;
     SL_REQUIRE(ws, SL_ERR_NULL);

@@ -38,6 +38,7 @@ __device__ __forceinline__ void load_code(const uint32_t *p, uint32_t (&c)[W]) {
 template <int W, int G_T, bool FUSED>
 __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     extern __shared__ uint32_t smem[];
+    __shared__ int s_range[2];  // smallest / largest score of this workgroup (fused flavour)
     const int b = blockIdx.y;
     const int KH = a.KH;
     const int G = G_T > 0 ? G_T : a.G;
@@ -78,6 +79,7 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     }
     if constexpr (FUSED) {
         for (int e = tid; e < KH * NB; e += HS_THREADS) hist[e] = 0;
+        if (tid == 0) { s_range[0] = NB - 1; s_range[1] = 0; }
     }
     if constexpr (FUSED || G_T == 0) __syncthreads();
 
@@ -95,6 +97,7 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     }
 
     const int full = G * W * 32;
+    int smin = NB - 1, smax = 0;
 #pragma unroll
     for (int u = 0; u < HS_U; ++u) {
         int dist = 0;
@@ -112,7 +115,11 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
         const int score = full - dist;  // matching bits
         const int64_t t = t0 + static_cast<int64_t>(u) * tok_per_pass + tl;
         if constexpr (FUSED) {
-            if (valid[u]) atomicAdd(&hist[h * NB + score], 1u);
+            if (valid[u]) {
+                atomicAdd(&hist[h * NB + score], 1u);
+                smin = score < smin ? score : smin;
+                smax = score > smax ? score : smax;
+            }
             sc_lds[h * (tok_per_pass * HS_U) + u * tok_per_pass + tl] =
                 static_cast<int16_t>(valid[u] ? score : 0);
         } else {
@@ -122,6 +129,15 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     }
 
     if constexpr (FUSED) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            smin = min(smin, __shfl_xor(smin, o, 64));
+            smax = max(smax, __shfl_xor(smax, o, 64));
+        }
+        if ((tid & 63) == 0) {
+            atomicMin(&s_range[0], smin);
+            atomicMax(&s_range[1], smax);
+        }
         __syncthreads();
         // head-major score rows: T int16 per head, four per lane
         const int T = tok_per_pass * HS_U;  // = 1024 / KH, a multiple of 4
@@ -134,12 +150,19 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
             *reinterpret_cast<uint2 *>(dst) = v;
         }
         // hist_groups copies of the global histogram spread the same-bin adds of the
-        // many workgroups of one (b, kv head) over as many addresses
+        // many workgroups of one (b, kv head) over as many addresses.  Only the
+        // bins between the smallest and largest score seen by this workgroup can
+        // be non-empty, so only those are visited.
+        const int lo = s_range[0], span = s_range[1] - lo + 1;
         const int grp = blockIdx.x % a.hist_groups;
-        for (int i = tid; i < KH * NB; i += HS_THREADS) {
-            const uint32_t c = hist[i];
-            const int hh = i / NB, bin = i % NB;
-            if (c) atomicAdd(&a.hist[((static_cast<int64_t>(b) * KH + hh) * a.hist_groups + grp) * NB + bin], c);
+        uint32_t *gh = a.hist + (static_cast<int64_t>(b) * KH * a.hist_groups + grp) * NB + lo;
+        for (int hh = 0; hh < KH; ++hh) {
+            const uint32_t *lh = hist + hh * NB + lo;
+            uint32_t *ghh = gh + static_cast<int64_t>(hh) * a.hist_groups * NB;
+            for (int i = tid; i < span; i += HS_THREADS) {
+                const uint32_t c = lh[i];
+                if (c) atomicAdd(&ghh[i], c);
+            }
         }
     }
 }
