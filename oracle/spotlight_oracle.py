@@ -464,3 +464,62 @@ def decode_step_reference_form(q, keys_rep, vals_rep, hash_weights, residue, mas
     out = torch.nn.functional.scaled_dot_product_attention(
         q, keys_rep, vals_rep, attn_mask=mask, is_causal=False)
     return out, idx
+
+
+# ---------------------------------------------------------------------------
+# The reference's patched attention forward, restated (torch, CPU)
+# ---------------------------------------------------------------------------
+
+def _rotate_half(x):
+    d = x.shape[-1]
+    return torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
+
+
+def reference_self_attn_forward(hidden_states, kv_cache, q_w, k_w, v_w, o_w, num_heads, num_kv_heads, hash_weights,
+                                residue, draft_enable, mask_out, min_remain, rope_theta=10000.0):
+    """spotlight_generation.py:109-226 step by step, for B == 1, on CPU.
+
+    q_w/k_w/v_w/o_w are the Linear weights ([out, in], no bias); hash_weights the
+    per-query-head [(proj [1,QH,in,out], bias [1,QH,1,out]), ...].  The cache holds
+    PRE-RoPE, repeat_kv'd keys and values; every call re-rotates the whole cache
+    (:139-141, modify_llama.py:68-80,103-113) and, when drafting, re-hashes it
+    (:14-17).  Returns (attn_output [1,t,hidden], kv_cache, indices or None)."""
+    B, t, hidden = hidden_states.shape
+    assert B == 1
+    d = hidden // num_heads
+    G = num_heads // num_kv_heads
+    is_prefill = t > 1 and kv_cache is None
+    ques = (hidden_states @ q_w.T).unflatten(-1, (num_heads, d)).transpose(1, 2)
+    keys = (hidden_states @ k_w.T).unflatten(-1, (num_kv_heads, d)).transpose(1, 2)
+    vals = (hidden_states @ v_w.T).unflatten(-1, (num_kv_heads, d)).transpose(1, 2)
+    keys = keys.repeat_interleave(G, dim=1)   # repeat_kv
+    vals = vals.repeat_interleave(G, dim=1)
+    if kv_cache is not None:
+        keys = torch.cat([kv_cache[0], keys], dim=-2)
+        vals = torch.cat([kv_cache[1], vals], dim=-2)
+    kv_cache = (keys, vals)
+    n = keys.shape[-2]
+    inv_freq = 1.0 / (rope_theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    ang = torch.arange(n, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    emb = torch.cat((ang, ang), dim=-1)
+    cos, sin = emb.cos().to(ques.dtype), emb.sin().to(ques.dtype)
+    rope = lambda m, p: m * cos[p][None, None] + _rotate_half(m) * sin[p][None, None]
+    Q = rope(ques, torch.arange(n - t, n))
+    Kr = rope(keys, torch.arange(n))
+    # causal base mask (modify_llama.py:132-143)
+    base = torch.full((1, 1, t, n), torch.finfo(Q.dtype).min, dtype=torch.float32)
+    base[0, 0, :, -t:].triu_(diagonal=1)
+    base[0, 0, :, :-t].fill_(0)
+    base = base.to(Q.dtype)
+    idx = None
+    mask = base
+    if draft_enable and not is_prefill:
+        sim = sign_matmul_score(mlp_hash_torch(Q, hash_weights, residue), mlp_hash_torch(Kr, hash_weights, residue))
+        k = num_remain(n, mask_out, min_remain)
+        idx = sim.topk(k=k, dim=-1).indices
+        m = torch.full((1, num_heads, t, n), torch.finfo(sim.dtype).min, dtype=sim.dtype)
+        m.scatter_(-1, idx, 0)
+        mask = torch.minimum(m, base)
+    out = torch.nn.functional.scaled_dot_product_attention(Q, Kr, vals, attn_mask=mask, is_causal=False)
+    out = out.transpose(1, 2).flatten(2) @ o_w.T
+    return out, kv_cache, idx

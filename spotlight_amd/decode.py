@@ -201,6 +201,27 @@ class LayerDecodeState:
             _lib.check(_L.sl_workspace_init(self.ws.data_ptr(), self.ws.numel(),
                                             torch.cuda.current_stream().cuda_stream), "sl_workspace_init")
 
+    def set_k(self, k: int) -> None:
+        """Tokens kept per (b, kv head) from the next step on (at most the k given at
+        construction, which sized the index buffers; rows of ``idx`` become k long).
+        The reference recomputes its budget from the cache length every step
+        (spotlight_generation.py:162-164)."""
+        if not 1 <= k <= self.k:
+            raise ValueError(f"k must be in [1, {self.k}]")
+        if self.lru_slots and k + 1 > self.lru_slots:
+            raise ValueError("k + 1 must not exceed the LRU slots")
+        self.params.k = k
+        self._graph = None
+
+    @property
+    def current_k(self) -> int:
+        return self.params.k
+
+    def selected(self) -> torch.Tensor:
+        """int32 [B, KH, current_k]: the tokens the last step attended to, ascending."""
+        k = self.params.k
+        return self.idx.view(-1)[: self.B * self.KH * k].view(self.B, self.KH, k)
+
     def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor) -> torch.Tensor:
         """One decode step: q [B,QH,d], k_new/v_new [B,KH,d] (post-RoPE).
         Returns the attention output [B,QH,d] (a buffer reused by the next step)."""

@@ -1,0 +1,236 @@
+"""Patched attention forward of the generation path, on the HIP kernels.
+
+Drop-in for the reference's ``self_attn_forward`` and the objects around it
+(spotlight/modifiers/spotlight_generation.py:109-226, 229-255, 298-330): same
+signature ``(self, hidden_states, kv_cache) -> (attn_output, kv_cache)``, same
+module attributes read (``config``, ``q_proj`` .. ``o_proj``, ``draft_kwargs``,
+``is_fix_layer``, ``hash_fn``), same hash-function parameter shapes, so a
+checkpoint written by the reference's ``Modifier.save_checkpoint``
+(spotlight/modifier.py:74-76) loads parameter for parameter.
+
+What differs is what happens to the cache, which callers treat as opaque
+(``model_model_forward`` only threads it through, :66-75):
+
+* keys are rotated ONCE, when they are appended, and stored post-RoPE with
+  their packed 128-bit code; the reference stores pre-RoPE keys and re-rotates
+  and re-hashes the whole cache every step (:139-141, :14-17);
+* K/V stay at kv-head granularity ``[B, n_cap, KH, d]``; the reference stores
+  them ``repeat_kv``-expanded (:128-136);
+* the decode branch (:143-215) runs as the fused HIP step instead of
+  sign-matmul + topk + mask + dense SDPA;
+* any batch size runs (the reference asserts B == 1, :138).
+
+Two ways to hash keys under GQA:
+  ``hash_fn_k`` present  -> one code per (token, kv head), scores summed over
+                            the G query heads of the group (the kernel path the
+                            reference's scorers are written for,
+                            spotlight/kernel/attn_dx_u32.py:68-128);
+  otherwise              -> ``per_qhead``: the cache is kept per query head
+                            (K/V repeated as the reference does) and every
+                            query head selects its own tokens with ``hash_fn``,
+                            which is exactly the reference's PyTorch path.
+"""
+from __future__ import annotations
+
+import json
+import math
+import types
+from typing import Optional
+
+import torch
+
+from .. import kernel as K
+from ..decode import HashWeights, LayerDecodeState
+
+
+class MLPLayer(torch.nn.Module):
+    """proj [1,H,in,out] ~ N(0,1)*0.001, bias [1,H,1,out] = 0 (spotlight_generation.py:229-240)."""
+
+    def __init__(self, info, num_heads, in_features, out_features, silu=False, residue=True):
+        super().__init__()
+        self.proj = torch.nn.Parameter(torch.randn((1, num_heads, in_features, out_features), **info) * 0.001)
+        self.bias = torch.nn.Parameter(torch.zeros((1, num_heads, 1, out_features), **info))
+        self.silu = torch.nn.SiLU() if silu else torch.nn.Identity()
+        self.resi = residue
+
+    def forward(self, x):
+        dx = self.silu(x @ self.proj + self.bias)
+        return dx + x if self.resi else dx
+
+
+class MLPHashingFunction(torch.nn.Module):
+    """spotlight_generation.py:243-255."""
+
+    def __init__(self, info, num_heads, num_mlp_layers, mlp_dims, mlp_residue):
+        super().__init__()
+        self.mlp = torch.nn.ModuleList(
+            MLPLayer(info, num_heads, mlp_dims[i], mlp_dims[i + 1], i < num_mlp_layers - 1, mlp_residue)
+            for i in range(num_mlp_layers))
+
+    def forward(self, x):
+        for module in self.mlp:
+            x = module(x)
+        return x
+
+    def hash_weights(self) -> HashWeights:
+        """The same parameters in the layout the kernels read ([H,in,out], [H,out])."""
+        layers = list(self.mlp)
+        if len(layers) not in (1, 2):
+            raise NotImplementedError("the fused hash kernel covers one or two layers")
+        w = [l.proj.data[0].contiguous() for l in layers]
+        b = [l.bias.data[0, :, 0].contiguous() for l in layers]
+        if len(layers) == 1:
+            return HashWeights(w[0], b[0], None, None, layers[0].resi)
+        return HashWeights(w[0], b[0], w[1], b[1], layers[0].resi)
+
+
+class LinearHashingFunction(torch.nn.Module):
+    """Gaussian projection x @ L (linearhashing_generation.py:224-231); the reference
+    hard-codes 32 heads of 128, here the head count is an argument."""
+
+    def __init__(self, info, num_heads=32, dim=128):
+        super().__init__()
+        self.linear = torch.nn.Parameter(torch.randn((1, num_heads, dim, dim), **info))
+
+    def forward(self, x):
+        return x @ self.linear
+
+    def hash_weights(self) -> HashWeights:
+        return HashWeights(self.linear.data[0].contiguous())
+
+
+def num_remain(n: int, mask_out: float, min_remain: int) -> int:
+    """spotlight_generation.py:162-164."""
+    return max(min(n, min_remain), n - int(n * mask_out))
+
+
+def rope_tables(positions: torch.Tensor, dim: int, theta: float, dtype) -> tuple:
+    """cos / sin [len, dim] for absolute positions, the rotate_half convention
+    (spotlight/modifiers/modify_llama.py:54-59 with transformers' rotary_emb)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, dim, 2, device=positions.device, dtype=torch.float32) / dim))
+    ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+    emb = torch.cat((ang, ang), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [B,t,H,d]; cos/sin [t,d]."""
+    d = x.shape[-1]
+    rot = torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
+    return x * cos[None, :, None, :] + rot * sin[None, :, None, :]
+
+
+class SpotlightKV:
+    """The per-layer cache handle threaded through the model in place of the
+    reference's ``(keys, vals)`` tuple."""
+
+    def __init__(self, B, QH, KH, d, n_cap, dtype, device, sparse_state: Optional[LayerDecodeState]):
+        self.B, self.QH, self.KH, self.d, self.n_cap = B, QH, KH, d, n_cap
+        self.state = sparse_state
+        if sparse_state is None:   # dense layer: plain K/V store
+            self.keys = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=device)
+            self.vals = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=device)
+        else:
+            self.keys, self.vals = sparse_state.keys, sparse_state.vals
+        self.length = 0
+
+    def append_dense(self, k, v):
+        t = k.shape[1]
+        if self.length + t > self.n_cap:
+            raise RuntimeError(f"cache capacity {self.n_cap} exceeded")
+        K.cache_append(self.keys, k.contiguous(), start=self.length)
+        K.cache_append(self.vals, v.contiguous(), start=self.length)
+        self.length += t
+
+
+def _dense_attention(q, keys, vals, causal):
+    """q [B,t,QH,d], keys/vals [B,n,KH,d] -> [B,t,QH,d]; torch SDPA with grouped heads."""
+    B, t, QH, d = q.shape
+    KH = keys.shape[2]
+    G = QH // KH
+    kk = keys.permute(0, 2, 1, 3).repeat_interleave(G, dim=1)
+    vv = vals.permute(0, 2, 1, 3).repeat_interleave(G, dim=1)
+    o = torch.nn.functional.scaled_dot_product_attention(q.permute(0, 2, 1, 3), kk, vv, is_causal=causal)
+    return o.permute(0, 2, 1, 3)
+
+
+def self_attn_forward(self, hidden_states: torch.Tensor, kv_cache=None):
+    """Same contract as spotlight_generation.py:109-226."""
+    cfg = self.config
+    QH, hidden = cfg.num_attention_heads, cfg.hidden_size
+    KH = cfg.num_key_value_heads
+    d = hidden // QH
+    B, t, _ = hidden_states.shape
+    dtype, dev = hidden_states.dtype, hidden_states.device
+    dk = self.draft_kwargs
+    sparse = dk.get("enable", True) is True and not self.is_fix_layer
+    per_qhead = getattr(self, "hash_fn_k", None) is None and KH != QH
+    G = QH // KH
+
+    ques = self.q_proj(hidden_states).unflatten(-1, (QH, d))
+    keys = self.k_proj(hidden_states).unflatten(-1, (KH, d))
+    vals = self.v_proj(hidden_states).unflatten(-1, (KH, d))
+
+    start = 0 if kv_cache is None else kv_cache.length
+    pos = torch.arange(start, start + t, device=dev)
+    cos, sin = rope_tables(pos, d, float(getattr(cfg, "rope_theta", 10000.0)), dtype)
+    ques = apply_rope(ques, cos, sin)
+    keys = apply_rope(keys, cos, sin)     # rotated once, here; stored post-RoPE
+    if sparse and per_qhead:              # the reference's repeat_kv (:128-129)
+        keys = keys.repeat_interleave(G, dim=2)
+        vals = vals.repeat_interleave(G, dim=2)
+    KHc = keys.shape[2]
+
+    if kv_cache is None:
+        n_cap = int(dk.get("max_cache_len", 0)) or (t + 1024)
+        n_cap = (max(n_cap, t + 1) + 7) // 8 * 8
+        state = None
+        if sparse:
+            hq = self.hash_fn.hash_weights()
+            hk = hq if per_qhead or KH == QH else self.hash_fn_k.hash_weights()
+            k_cap = num_remain(n_cap, dk["mask_out"], dk["min_remain"])
+            state = LayerDecodeState(B, QH, KHc, d, n_cap, k_cap, hq, hk,
+                                     dtype=dtype, device=dev, head_map="blocked")
+        kv_cache = SpotlightKV(B, QH, KHc, d, n_cap, dtype, dev, state)
+
+    if t > 1 or not sparse or kv_cache.length == 0:
+        # prefill (the draft is not used there, :145) and dense layers
+        if kv_cache.state is not None:
+            if kv_cache.length != 0:
+                raise NotImplementedError("chunked prefill of a sparse layer")
+            kv_cache.state.prefill(keys.contiguous(), vals.contiguous())
+            kv_cache.length = t
+        else:
+            kv_cache.append_dense(keys, vals)
+        n = kv_cache.length
+        out = _dense_attention(ques, kv_cache.keys[:, :n], kv_cache.vals[:, :n], causal=t > 1)
+    else:
+        st = kv_cache.state
+        n = kv_cache.length + 1
+        k = num_remain(n, dk["mask_out"], dk["min_remain"])
+        if k != st.current_k:
+            st.set_k(k)
+        out = st.step(ques[:, 0].contiguous(), keys[:, 0].contiguous(), vals[:, 0].contiguous()).unsqueeze(1)
+        kv_cache.length = n
+
+    attn_output = self.o_proj(out.reshape(B, t, hidden))
+    return attn_output, kv_cache
+
+
+def patch_attention(attn_module: torch.nn.Module, layer_idx: int, draft_kwargs: dict,
+                    gqa_key_hash: bool = False) -> None:
+    """What Decoder.__init__ does to every layer's attention (spotlight_generation.py:317-329):
+    install draft_kwargs / is_fix_layer / hash_fn and bind the forward.  With
+    ``gqa_key_hash`` a second, per-kv-head hash function ``hash_fn_k`` is created."""
+    cfg = attn_module.config
+    info = {"device": attn_module.q_proj.weight.data.device, "dtype": attn_module.q_proj.weight.data.dtype}
+    mlp_dims = draft_kwargs.get("mlp_dims", "[128,128,128]")
+    mlp_dims = json.loads(mlp_dims) if isinstance(mlp_dims, str) else list(mlp_dims)
+    n_layers = draft_kwargs.get("num_mlp_layers", 2)
+    residue = draft_kwargs.get("mlp_residue", True)
+    attn_module.is_fix_layer = layer_idx in draft_kwargs.get("fix_layers", [])
+    attn_module.draft_kwargs = draft_kwargs
+    attn_module.hash_fn = MLPHashingFunction(info, cfg.num_attention_heads, n_layers, mlp_dims, residue)
+    if gqa_key_hash and cfg.num_key_value_heads != cfg.num_attention_heads:
+        attn_module.hash_fn_k = MLPHashingFunction(info, cfg.num_key_value_heads, n_layers, mlp_dims, residue)
+    attn_module.forward = types.MethodType(self_attn_forward, attn_module)
