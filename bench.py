@@ -71,6 +71,8 @@ def main():
     ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch heuristic passed to sl_tune (e.g. attn_target_wgs=128)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (reference point for HBM byte counters)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-breakdown", action="store_true")
     args = ap.parse_args()
@@ -176,6 +178,14 @@ def main():
     us_per_step = ms_per_step * 1e3
     n_mid = n0 + (math.ceil(warmup / L) + steps / L / 2)
     ab = algorithmic_bytes(c, n_mid)
+
+    if args.calibration_copy:
+        src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- per-kernel durations: HIP events around a graph of M launches of one stage, rotating layers
     kernels = {}

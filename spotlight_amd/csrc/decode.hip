@@ -75,7 +75,8 @@ extern "C" int sl_version(void) { return 100; }
 
 extern "C" int sl_tune(const char *key, int value) {
     SL_REQUIRE(key, SL_ERR_NULL);
-    return sl_attn_tune(key, value);
+    const int rc = sl_attn_tune(key, value);
+    return rc == SL_OK ? rc : sl_select_tune(key, value);
 }
 
 extern "C" int sl_workspace_init(void *ws, size_t ws_bytes, void *stream) {

@@ -2,7 +2,7 @@
 #pragma once
 #include "common.h"
 
-constexpr int TK_THREADS = 256;
+constexpr int TK_THREADS = 1024;
 constexpr int TK_MAX_BINS = 4608;
 
 struct select_args {
@@ -24,3 +24,4 @@ size_t sl_select_ws_bytes(int B, int KH, int n_bins, int64_t n);
 // points hist / thr_need / block_cnt of `a` into `ws` (a.B, a.KH, a.n_bins set)
 void sl_select_carve(select_args &a, void *ws, int64_t n_for_blocks);
 int sl_select_launch(const select_args &a, hipStream_t s);
+int sl_select_tune(const char *key, int value);

@@ -15,8 +15,8 @@
 //      threshold resolve to the lowest token index.  No sort, no atomics in
 //      the selection, and the result is the same on every run.
 //
-// Work is cut into blocks of 2048 tokens, one workgroup per (block, b, kv
-// head): a compute unit needs some 20 instructions per token, so one
+// Work is cut into blocks of 8192 tokens, one workgroup of 16 waves per (block,
+// b, kv head): a compute unit needs some 20 instructions per token, so one
 // workgroup per (b, kv head) would spend microseconds per 10k tokens.  Every
 // workgroup derives (thr, need) itself (the histogram is 2 KB).  What it also
 // needs is the number of tokens above / at the threshold in the blocks before
@@ -28,12 +28,14 @@
 //     sums them (select_count_kernel + select_compact_kernel).
 #include "topk.h"
 
+#include <string.h>
+
 namespace {
 
 constexpr int TK_RUN = 8;                          // consecutive tokens per lane (one 16-byte load)
 constexpr int TK_BLOCK = TK_THREADS * TK_RUN;      // tokens per workgroup
 constexpr int TK_MAX_BPT = (TK_MAX_BINS + TK_THREADS - 1) / TK_THREADS;  // histogram bins a lane owns
-constexpr int TK_FUSE_BLOCKS = 32;                 // single-launch path up to this many blocks
+constexpr int TK_FUSE_BLOCKS = 16;                 // single-launch path up to this many blocks (and <= 1024 bins)
 
 __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *p, int64_t n) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -270,9 +272,9 @@ __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a)
         for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;
     if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b) return;
     if (blk == 0) select_fused_body<CONTIG, MAX_BPT, NG, 0>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
+    else if (blk <= 1) select_fused_body<CONTIG, MAX_BPT, NG, 1>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
     else if (blk <= 3) select_fused_body<CONTIG, MAX_BPT, NG, 3>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
     else if (blk <= 7) select_fused_body<CONTIG, MAX_BPT, NG, 7>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
-    else if (blk <= 15) select_fused_body<CONTIG, MAX_BPT, NG, 15>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
     else select_fused_body<CONTIG, MAX_BPT, NG, TK_FUSE_BLOCKS - 1>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
 }
 
@@ -342,7 +344,15 @@ __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args 
 
 }  // namespace
 
+static int g_hist_copies = 0;  // sl_tune("hist_copies", 4 | 16); 0 = by cache length
+
+int sl_select_tune(const char *key, int value) {
+    if (!strcmp(key, "hist_copies") && (value == 0 || value == 4 || value == 16)) { g_hist_copies = value; return SL_OK; }
+    return SL_ERR_UNSUPPORTED;
+}
+
 int sl_select_hist_groups(int64_t n) {
+    if (g_hist_copies) return g_hist_copies;
     // Copies of every histogram bin, so that the same-bin adds of the many scorer
     // workgroups of one (b, kv head) spread over as many addresses: 16 for long
     // caches, 4 for short ones (fewer workgroups, and the copies must be cleared
@@ -382,12 +392,12 @@ int sl_select_launch(const select_args &a, hipStream_t s) {
     const bool contig = a.stride_n == 1 && sl_aligned(a.score, 16) && a.stride_b % 8 == 0 && a.stride_h % 8 == 0 &&
                         a.stride_h >= (a.n + 7) / 8 * 8;
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(bh));
-    const bool small = a.n_bins <= 4 * TK_THREADS;  // few bins per lane: the common case
+    const bool small = a.n_bins <= TK_THREADS;  // one bin per lane: the common case (G * nbits <= 1023)
     SL_REQUIRE(a.hist_groups == 4 || a.hist_groups == 16, SL_ERR_UNSUPPORTED);
 #define SL_SELECT_LAUNCH(CONTIG, BPT, NG)                                                        \
     do {                                                                                         \
-        if (blocks <= TK_FUSE_BLOCKS) {                                                          \
-            select_fused_kernel<CONTIG, BPT, NG><<<grid, dim3(TK_THREADS), 0, s>>>(a);           \
+        if (CONTIG && BPT == 1 && blocks <= TK_FUSE_BLOCKS) { /* strided scores: two launches */ \
+            select_fused_kernel<true, 1, NG><<<grid, dim3(TK_THREADS), 0, s>>>(a);               \
         } else {                                                                                 \
             select_count_kernel<CONTIG, BPT, NG><<<grid, dim3(TK_THREADS), 0, s>>>(a);           \
             select_compact_kernel<CONTIG><<<grid, dim3(TK_THREADS), 0, s>>>(a);                  \
@@ -399,10 +409,10 @@ int sl_select_launch(const select_args &a, hipStream_t s) {
         else SL_SELECT_LAUNCH(CONTIG, BPT, 4);                    \
     } while (0)
     if (contig) {
-        if (small) SL_SELECT_NG(true, 4);
+        if (small) SL_SELECT_NG(true, 1);
         else SL_SELECT_NG(true, TK_MAX_BPT);
     } else {
-        if (small) SL_SELECT_NG(false, 4);
+        if (small) SL_SELECT_NG(false, 1);
         else SL_SELECT_NG(false, TK_MAX_BPT);
     }
 #undef SL_SELECT_NG
