@@ -194,7 +194,8 @@ def main():
         # equalise lengths (a partial token may have advanced only some layers)
         M = 4 * L
         stage_sets = [("hash", _lib.STAGE_HASH), ("score", _lib.STAGE_SCORE),
-                      ("score+select", _lib.STAGE_SCORE | _lib.STAGE_SELECT), ("attn", _lib.STAGE_ATTN)]
+                      ("score+select", _lib.STAGE_SCORE | _lib.STAGE_SELECT), ("attn", _lib.STAGE_ATTN),
+                      ("select+attn", _lib.STAGE_SELECT | _lib.STAGE_ATTN)]
         if c["lru"]:
             stage_sets.insert(3, ("lru", _lib.STAGE_LRU))
         raw = {}
@@ -212,17 +213,20 @@ def main():
             torch.cuda.synchronize()
             raw[name] = e0.elapsed_time(e1) * 1e3 / M
             del g
-            if name == "score":
-                for st in layers:
-                    st.reset_workspace()
-                torch.cuda.synchronize()
         raw["select"] = max(raw["score+select"] - raw["score"], 0.0)
-        for name in ("hash", "score", "select", "lru", "attn"):
+        ab["select+attn"] = ab["attn"]
+        # the step runs selection and attention as one launch when it can (no LRU, <= 64k rows):
+        # then "select+attn" is that launch and "select" / "attn" are the two-launch alternative
+        fused_tail = not c["lru"] and raw["select+attn"] < 0.9 * (raw["select"] + raw["attn"])
+        names = ("hash", "score", "select+attn") if fused_tail else ("hash", "score", "select", "lru", "attn")
+        for name in ("hash", "score", "select", "lru", "attn", "select+attn"):
             if name in raw:
                 us = raw[name]
                 kernels[name] = {"us": round(us, 3), "algorithmic_bytes": ab[name],
-                                 "gbps": round(ab[name] / us / 1e3, 1) if us > 0 else None}
-        dominant = max((n for n in kernels if kernels[n]["algorithmic_bytes"] > 0), key=lambda n: kernels[n]["us"])
+                                 "gbps": round(ab[name] / us / 1e3, 1) if us > 0 else None,
+                                 "in_step": name in names}
+        dominant = max((n for n in kernels if kernels[n]["in_step"] and kernels[n]["algorithmic_bytes"] > 0),
+                       key=lambda n: kernels[n]["us"])
 
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")

@@ -18,5 +18,7 @@ struct attn_args {
 };
 
 size_t sl_attn_ws_bytes(int B, int QH, int KH, int k);
+// points counter / part of `a` into the workspace and fills in the default scale
+int sl_attn_prepare(attn_args &a, void *ws, size_t ws_bytes);
 int sl_attn_launch(attn_args a, void *ws, size_t ws_bytes, hipStream_t s);
 int sl_attn_tune(const char *key, int value);

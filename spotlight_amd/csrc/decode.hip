@@ -8,12 +8,17 @@
 //                        threshold from the histogram, stable compaction -> idx
 //   4. lru_kernel        (optional) resident-table update -> slot list
 //   5. sparse_attn_kernel over idx (or over the resident slots), then seq_lens[b] += 1
+//   (3 and 5 run as ONE launch, select_attend_kernel, when there is no LRU and the cache
+//    has at most 64k rows)
 // Every length is read from device memory, so the same captured HIP graph can
 // be replayed while the cache grows.
+#include <string.h>
+
 #include "attn.h"
 #include "hamming.h"
 #include "hash.h"
 #include "lru.h"
+#include "select_attend.h"
 #include "topk.h"
 
 namespace {
@@ -24,6 +29,8 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, ui
     for (size_t j = i; j < n16; j += stride) p[j] = make_uint4(0, 0, 0, 0);
     if (i < n_tail) tail[i] = 0;
 }
+
+int g_fuse_select_attend = 1;  // sl_tune("fuse_select_attend", 0 | 1)
 
 struct ws_layout {
     size_t q_code, select, score, attn, total;
@@ -75,6 +82,7 @@ extern "C" int sl_version(void) { return 100; }
 
 extern "C" int sl_tune(const char *key, int value) {
     SL_REQUIRE(key, SL_ERR_NULL);
+    if (!strcmp(key, "fuse_select_attend")) { g_fuse_select_attend = value != 0; return SL_OK; }
     const int rc = sl_attn_tune(key, value);
     return rc == SL_OK ? rc : sl_select_tune(key, value);
 }
@@ -159,17 +167,24 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     ta.score = score; ta.idx = p.idx; ta.seq_lens = p.seq_lens;
     ta.k = p.k; ta.len_bias = 1; ta.n = p.n_max;
     ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
+    // 3. select -- or 3+5 in one launch when there is no LRU in between and the shapes allow
+    attn_args aa{};
+    aa.q = p.q; aa.out = p.out; aa.dtype = p.dtype; aa.B = p.B; aa.QH = p.QH; aa.KH = p.KH; aa.k = p.k;
+    aa.rows = 0; aa.scale = 0.f; aa.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
+    const bool whole = stages == SL_STAGE_ALL;  // lengths only advance on a complete step
+    aa.bump_lens = whole ? p.seq_lens : nullptr; aa.bump_step = whole ? p.step_counter : nullptr;
+    aa.keys = p.keys; aa.vals = p.vals; aa.idx = p.idx;
+    aa.kv_stride_b = p.n_cap * p.KH * p.d; aa.kv_stride_h = p.d;
+    aa.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
+    const bool both = (stages & SL_STAGE_SELECT) && (stages & SL_STAGE_ATTN);
+    if (both && p.lru_C == 0 && g_fuse_select_attend && sl_select_attend_supported(ta, aa))
+        return sl_select_attend_launch(ta, aa, ws + L.attn, L.total - L.attn, s);
     if (stages & SL_STAGE_SELECT) {
         rc = sl_select_launch(ta, s);
         if (rc != SL_OK) return rc;
     }
 
     // 4. optional LRU, 5. attention
-    attn_args aa{};
-    aa.q = p.q; aa.out = p.out; aa.dtype = p.dtype; aa.B = p.B; aa.QH = p.QH; aa.KH = p.KH; aa.k = p.k;
-    aa.rows = 0; aa.scale = 0.f; aa.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
-    const bool whole = stages == SL_STAGE_ALL;  // lengths only advance on a complete step
-    aa.bump_lens = whole ? p.seq_lens : nullptr; aa.bump_step = whole ? p.step_counter : nullptr;
     if (p.lru_C > 0) {
         SL_REQUIRE(p.k + 1 <= p.lru_C && p.lru_C <= LRU_MAX_SLOTS, SL_ERR_UNSUPPORTED);
         lru_args la{};
@@ -186,10 +201,6 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         aa.kv_stride_b = static_cast<int64_t>(p.KH) * p.lru_C * p.d;
         aa.kv_stride_h = static_cast<int64_t>(p.lru_C) * p.d;
         aa.kv_stride_n = p.d;
-    } else {
-        aa.keys = p.keys; aa.vals = p.vals; aa.idx = p.idx;
-        aa.kv_stride_b = p.n_cap * p.KH * p.d; aa.kv_stride_h = p.d;
-        aa.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
     }
     if (!(stages & SL_STAGE_ATTN)) return SL_OK;
     return sl_attn_launch(aa, ws + L.attn, L.total - L.attn, s);

@@ -1,0 +1,134 @@
+// Fused count-select + sparse attention: the last two stages of the decode step
+// in one launch.
+//
+// One workgroup of 8 waves per 4096-token block of a (b, kv head).  It derives
+// (thr, need) from the histogram, counts the blocks before its own, places its
+// kept tokens -- into the global index list AND into an LDS list -- and then
+// attends over exactly those rows (attn_core.h), as run `block` of the
+// (b, kv head).  Compared with select + attention as two launches this removes
+// one launch and the store -> load round trip of the index list; the runs are
+// token ranges instead of rank ranges, so a (b, kv head) whose kept tokens
+// cluster in one block is served by fewer workgroups (the result is the same).
+// Used for up to 16 blocks (64k tokens) and up to 1024 score bins.
+#include "select_attend.h"
+
+#include "attn_core.h"
+#include "topk_core.h"
+
+namespace {
+
+constexpr int SA_NW = 8;
+constexpr int SA_THREADS = SA_NW * 64;
+constexpr int SA_BLOCK = SA_THREADS * TK_RUN;   // 4096 tokens
+constexpr int SA_U = 2;                         // row groups in flight per iteration (64 rows per workgroup)
+constexpr int SA_MAX_BPT = 2;                   // histogram bins per lane (<= 1024 bins)
+
+template <bool dummy = true> struct sa_static_checks {
+    static_assert(SA_MAX_BLOCKS == AT_MAX_SPLITS, "one attention run per token block");
+};
+
+template <int NG, int NPREV>
+__device__ __forceinline__ void sa_select(const select_args &a, int blk, int bh, int b, int h, int64_t n_b, int k_eff,
+                                          int32_t *out, uint32_t *s_wave, int *s_tn, int32_t *s_list, int *n_kept) {
+    const int tid = threadIdx.x;
+    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
+    const int64_t t0 = static_cast<int64_t>(blk) * SA_BLOCK + tid * TK_RUN;
+    const uint4 v = load_run<true>(a, sc, t0, n_b);
+    uint4 prev[NPREV > 0 ? NPREV : 1];
+#pragma unroll
+    for (int j = 0; j < NPREV; ++j)
+        prev[j] = load_run<true>(a, sc, static_cast<int64_t>(j < blk ? j : blk) * SA_BLOCK + tid * TK_RUN, n_b);
+    uint32_t cnt[SA_MAX_BPT];
+    const uint32_t mine = load_bins<SA_THREADS, SA_MAX_BPT, NG>(a, bh, cnt);
+    int thr, need;
+    find_threshold<SA_THREADS, SA_MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+    uint32_t pg = 0, pe = 0;
+#pragma unroll
+    for (int j = 0; j < NPREV; ++j) {
+        const uint32_t c = j < blk ? count_run(prev[j], thr) : 0u;
+        pg += c & 0xffffu;
+        pe += c >> 16;
+    }
+    uint32_t tg, te;
+    block_exclusive_sum<SA_THREADS>(pg, s_wave, &tg);
+    __syncthreads();
+    block_exclusive_sum<SA_THREADS>(pe, s_wave, &te);
+    __syncthreads();
+    place_block<SA_THREADS, true>(v, t0, thr, need, k_eff, tg, te, s_wave, out, s_list, n_kept);
+}
+
+template <typename T, int G, int NG>
+__global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args sa, attn_args aa) {
+    __shared__ uint32_t s_wave[SA_THREADS / 64 + 1];
+    __shared__ int s_tn[2];
+    __shared__ int32_t s_list[SA_BLOCK + SA_NW * 4 * SA_U];
+    __shared__ attn_shared<G, SA_NW> sh;
+
+    const int tid = threadIdx.x;
+    const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int bh = b * sa.KH + h;
+    const int64_t n_b = tokens_of(sa, b);
+    const int k_eff = n_b < sa.k ? static_cast<int>(n_b) : sa.k;
+    int32_t *out = sa.idx + static_cast<int64_t>(bh) * sa.k;
+    if (blk == 0)
+        for (int i = k_eff + tid; i < sa.k; i += SA_THREADS) out[i] = -1;
+    if (static_cast<int64_t>(blk) * SA_BLOCK >= n_b) return;
+    const int S = static_cast<int>((n_b + SA_BLOCK - 1) / SA_BLOCK);  // runs of this (b, kv head)
+
+    int n_kept = 0;
+    if (blk == 0) sa_select<NG, 0>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
+    else if (blk <= 1) sa_select<NG, 1>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
+    else if (blk <= 3) sa_select<NG, 3>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
+    else if (blk <= 7) sa_select<NG, 7>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
+    else sa_select<NG, SA_MAX_BLOCKS - 1>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
+
+    // pad the list to whole iterations of the attention loop, then attend over it
+    constexpr int ITER = SA_NW * 4 * SA_U;
+    const int padded = (n_kept + ITER - 1) / ITER * ITER;
+    __syncthreads();
+    for (int i = n_kept + tid; i < padded; i += SA_THREADS) s_list[i] = -1;
+    __syncthreads();
+    attend_rows_and_merge<T, G, SA_NW, SA_U>(aa, b, h, blk, S, s_list, n_kept, sh);
+}
+
+template <typename T, int G>
+int launch_ng(const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
+    if (sa.hist_groups == 16) select_attend_kernel<T, G, 16><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
+    else select_attend_kernel<T, G, 4><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
+    return sl_check_launch();
+}
+
+template <typename T>
+int launch_g(const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
+    switch (aa.QH / aa.KH) {
+        case 1: return launch_ng<T, 1>(sa, aa, grid, s);
+        case 2: return launch_ng<T, 2>(sa, aa, grid, s);
+        case 4: return launch_ng<T, 4>(sa, aa, grid, s);
+        default: return SL_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace
+
+bool sl_select_attend_supported(const select_args &sa, const attn_args &aa) {
+    const int G = aa.QH / aa.KH;
+    const int64_t blocks = (sa.n + SA_BLOCK - 1) / SA_BLOCK;
+    return (G == 1 || G == 2 || G == 4) && blocks <= SA_MAX_BLOCKS && sa.n_bins <= SA_THREADS * SA_MAX_BPT &&
+           (sa.hist_groups == 4 || sa.hist_groups == 16) && sa.stride_n == 1 && sa.stride_b % 8 == 0 &&
+           sa.stride_h % 8 == 0 && sa.stride_h >= (sa.n + 7) / 8 * 8 && sl_aligned(sa.score, 16) && aa.B <= 65535;
+}
+
+int sl_select_attend_launch(const select_args &sa, attn_args aa, void *attn_ws, size_t attn_ws_bytes, hipStream_t s) {
+    SL_REQUIRE(sl_select_attend_supported(sa, aa), SL_ERR_UNSUPPORTED);
+    int rc = sl_attn_prepare(aa, attn_ws, attn_ws_bytes);
+    if (rc != SL_OK) return rc;
+    int64_t blocks = (sa.n + SA_BLOCK - 1) / SA_BLOCK;
+    if (blocks < 1) blocks = 1;
+    const dim3 grid(static_cast<unsigned>(blocks), sa.KH, sa.B);
+    switch (aa.dtype) {
+        case SL_F32: return launch_g<float>(sa, aa, grid, s);
+        case SL_BF16: return launch_g<bf16_t>(sa, aa, grid, s);
+        case SL_F16: return launch_g<f16_t>(sa, aa, grid, s);
+        default: return SL_ERR_UNSUPPORTED;
+    }
+}

@@ -26,13 +26,12 @@
 //     one launch (select_fused_kernel);
 //   * beyond that, a first launch writes per-block counts and a second one
 //     sums them (select_count_kernel + select_compact_kernel).
-#include "topk.h"
+#include "topk_core.h"
 
 #include <string.h>
 
 namespace {
 
-constexpr int TK_RUN = 8;                          // consecutive tokens per lane (one 16-byte load)
 constexpr int TK_BLOCK = TK_THREADS * TK_RUN;      // tokens per workgroup
 constexpr int TK_MAX_BPT = (TK_MAX_BINS + TK_THREADS - 1) / TK_THREADS;  // histogram bins a lane owns
 constexpr int TK_FUSE_BLOCKS = 16;                 // single-launch path up to this many blocks (and <= 1024 bins)
@@ -47,15 +46,6 @@ __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *p, int64_t n)
 // LDS); LDS histogram per head, then flush.
 constexpr int SH_THREADS = 256;
 constexpr int SH_TOKENS = 512;  // tokens per workgroup
-
-__device__ __forceinline__ int64_t tokens_of(const select_args &a, int b) {
-    int64_t n_b = a.n;
-    if (a.seq_lens) {
-        const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
-        n_b = l < n_b ? l : n_b;
-    }
-    return n_b;
-}
 
 __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, int heads_per_group) {
     extern __shared__ uint32_t hist[];
@@ -88,138 +78,6 @@ __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, i
     }
 }
 
-// ---- pieces shared by the select kernels ---------------------------------------
-
-// Eight consecutive scores of one lane as four packed words (token 2j in the low
-// half of word j).  The load is unconditional and branch free: CONTIG reads the
-// 16 bytes at t0 (callers guarantee they lie inside the allocation), the strided
-// flavour clamps each token index; tokens at or beyond n_b then become -1, which
-// never qualifies.
-template <bool CONTIG>
-__device__ __forceinline__ uint4 load_run(const select_args &a, const int16_t *sc, int64_t t0, int64_t n_b) {
-    uint32_t w[4];
-    if constexpr (CONTIG) {
-        const uint4 r = *reinterpret_cast<const uint4 *>(sc + t0);
-        w[0] = r.x; w[1] = r.y; w[2] = r.z; w[3] = r.w;
-    } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int64_t t = t0 + 2 * j;
-            const int64_t last = n_b > 0 ? n_b - 1 : 0;
-            const uint32_t lo = static_cast<uint16_t>(sc[(t < last ? t : last) * a.stride_n]);
-            const uint32_t hi = static_cast<uint16_t>(sc[(t + 1 < last ? t + 1 : last) * a.stride_n]);
-            w[j] = lo | (hi << 16);
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int64_t t = t0 + 2 * j;
-        if (t >= n_b) w[j] |= 0xffffu;
-        if (t + 1 >= n_b) w[j] |= 0xffff0000u;
-    }
-    return make_uint4(w[0], w[1], w[2], w[3]);
-}
-
-__device__ __forceinline__ void unpack_run(const uint4 &r, int (&v)[TK_RUN]) {
-    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        v[2 * j] = static_cast<int16_t>(w[j] & 0xffffu);
-        v[2 * j + 1] = static_cast<int16_t>(w[j] >> 16);
-    }
-}
-
-// Lane `tid` owns bins NB-1 - (tid*BPT + j), best scores first, and sums their NG
-// copies; every load of the lane is independent of the others (one round trip).
-template <int MAX_BPT, int NG>
-__device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, uint32_t (&cnt)[MAX_BPT]) {
-    const int NB = a.n_bins, tid = threadIdx.x;
-    const int BPT = (NB + TK_THREADS - 1) / TK_THREADS;
-    const uint32_t *gh = a.hist + static_cast<int64_t>(bh) * NG * NB;
-    uint32_t raw[MAX_BPT][NG];
-#pragma unroll
-    for (int j = 0; j < MAX_BPT; ++j) {
-        const int bi = tid * BPT + j;
-        const bool live = j < BPT && bi < NB;
-        const int bin = live ? NB - 1 - bi : 0;  // unconditional loads, dead bins are dropped below
-#pragma unroll
-        for (int g = 0; g < NG; ++g) raw[j][g] = gh[g * NB + bin];
-    }
-    uint32_t mine = 0;
-#pragma unroll
-    for (int j = 0; j < MAX_BPT; ++j) {
-        const int bi = tid * BPT + j;
-        uint32_t c = 0;
-#pragma unroll
-        for (int g = 0; g < NG; ++g) c += raw[j][g];
-        cnt[j] = (j < BPT && bi < NB) ? c : 0u;
-        mine += cnt[j];
-    }
-    return mine;
-}
-
-// Block-wide search of the threshold bin; every lane returns (thr, need).
-template <int MAX_BPT>
-__device__ __forceinline__ void find_threshold(const select_args &a, const uint32_t (&cnt)[MAX_BPT],
-                                               uint32_t mine, int k_eff, uint32_t *s_wave, int *s_tn,
-                                               int &thr, int &need) {
-    const int NB = a.n_bins, tid = threadIdx.x;
-    const int BPT = (NB + TK_THREADS - 1) / TK_THREADS;
-    if (tid == 0) { s_tn[0] = NB; s_tn[1] = 0; }  // selects nothing unless a lane finds the bin
-    uint32_t total;
-    uint32_t cum = block_exclusive_sum<TK_THREADS>(mine, s_wave, &total);
-#pragma unroll
-    for (int j = 0; j < MAX_BPT; ++j) {
-        if (k_eff > 0 && cum < static_cast<uint32_t>(k_eff) && cum + cnt[j] >= static_cast<uint32_t>(k_eff)) {
-            s_tn[0] = NB - 1 - (tid * BPT + j);
-            s_tn[1] = k_eff - static_cast<int>(cum);
-        }
-        cum += cnt[j];
-    }
-    __syncthreads();
-    thr = s_tn[0];
-    need = s_tn[1];
-}
-
-__device__ __forceinline__ uint32_t count_run(const uint4 &r, int thr) {
-    int v[TK_RUN];
-    unpack_run(r, v);
-    uint32_t gt = 0, eq = 0;
-#pragma unroll
-    for (int j = 0; j < TK_RUN; ++j) {
-        gt += v[j] > thr;
-        eq += v[j] == thr;
-    }
-    return gt | (eq << 16);
-}
-
-// Places the kept tokens of one block.  (tg, te): tokens above / at the threshold
-// in all earlier blocks.  Contains barriers.
-__device__ __forceinline__ void place_block(const uint4 &run, int64_t t0, int thr, int need, int k_eff,
-                                            uint32_t tg, uint32_t te, uint32_t *s_wave, int32_t *out) {
-    const uint32_t uneed = static_cast<uint32_t>(need);
-    uint32_t tot;
-    const uint32_t ex = block_exclusive_sum<TK_THREADS>(count_run(run, thr), s_wave, &tot);
-    int v[TK_RUN];
-    unpack_run(run, v);
-    uint32_t gt_before = tg + (ex & 0xffffu), eq_before = te + (ex >> 16);
-#pragma unroll
-    for (int j = 0; j < TK_RUN; ++j) {
-        const int s = v[j];
-        if (s > thr) {
-            const uint32_t pos = gt_before + (eq_before < uneed ? eq_before : uneed);
-            if (pos < static_cast<uint32_t>(k_eff)) out[pos] = static_cast<int32_t>(t0 + j);
-            ++gt_before;
-        } else if (s == thr) {
-            if (eq_before < uneed) {
-                const uint32_t pos = gt_before + eq_before;
-                if (pos < static_cast<uint32_t>(k_eff)) out[pos] = static_cast<int32_t>(t0 + j);
-            }
-            ++eq_before;
-        }
-    }
-}
-
 // ---- single launch: every block counts the blocks before it ---------------------
 
 // Body for a block with at most NPREV blocks before it: the NPREV loads are
@@ -236,10 +94,10 @@ __device__ __forceinline__ void select_fused_body(const select_args &a, int blk,
     for (int j = 0; j < NPREV; ++j)
         prev[j] = load_run<CONTIG>(a, sc, static_cast<int64_t>(j < blk ? j : blk) * TK_BLOCK + tid * TK_RUN, n_b);
     uint32_t cnt[MAX_BPT];
-    const uint32_t mine = load_bins<MAX_BPT, NG>(a, bh, cnt);
+    const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, cnt);
 
     int thr, need;
-    find_threshold<MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
 
     uint32_t pg = 0, pe = 0;
 #pragma unroll
@@ -255,7 +113,7 @@ __device__ __forceinline__ void select_fused_body(const select_args &a, int blk,
     __syncthreads();
     const uint32_t uneed = static_cast<uint32_t>(need);
     if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
-    place_block(v, t0, thr, need, k_eff, tg, te, s_wave, out);
+    place_block<TK_THREADS>(v, t0, thr, need, k_eff, tg, te, s_wave, out);
 }
 
 template <bool CONTIG, int MAX_BPT, int NG>
@@ -295,9 +153,9 @@ __global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a)
     const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
     const uint4 v = load_run<CONTIG>(a, sc, t0, n_b);
     uint32_t cnt[MAX_BPT];
-    const uint32_t mine = load_bins<MAX_BPT, NG>(a, bh, cnt);
+    const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, cnt);
     int thr, need;
-    find_threshold<MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
     if (blk == 0 && tid == 0) {
         a.thr_need[bh * 2] = thr;
         a.thr_need[bh * 2 + 1] = need;
@@ -339,7 +197,7 @@ __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args 
     __syncthreads();
     const uint32_t uneed = static_cast<uint32_t>(need);
     if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
-    place_block(v, t0, thr, need, k_eff, tg, te, s_wave, out);
+    place_block<TK_THREADS>(v, t0, thr, need, k_eff, tg, te, s_wave, out);
 }
 
 }  // namespace

@@ -1,0 +1,164 @@
+// Device-side pieces of the count-select, shared by the select kernels and the
+// fused select + attend kernel.  NT = lanes per workgroup; a workgroup owns a
+// block of NT * 8 consecutive tokens of one (b, kv head).
+#pragma once
+#include "topk.h"
+
+constexpr int TK_RUN = 8;  // consecutive tokens per lane (one 16-byte load)
+
+__device__ __forceinline__ int64_t tokens_of(const select_args &a, int b) {
+    int64_t n_b = a.n;
+    if (a.seq_lens) {
+        const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
+        n_b = l < n_b ? l : n_b;
+    }
+    return n_b;
+}
+
+// ---- pieces shared by the select kernels ---------------------------------------
+
+// Eight consecutive scores of one lane as four packed words (token 2j in the low
+// half of word j).  The load is unconditional and branch free: CONTIG reads the
+// 16 bytes at t0 (callers guarantee they lie inside the allocation), the strided
+// flavour clamps each token index; tokens at or beyond n_b then become -1, which
+// never qualifies.
+template <bool CONTIG>
+__device__ __forceinline__ uint4 load_run(const select_args &a, const int16_t *sc, int64_t t0, int64_t n_b) {
+    uint32_t w[4];
+    if constexpr (CONTIG) {
+        const uint4 r = *reinterpret_cast<const uint4 *>(sc + t0);
+        w[0] = r.x; w[1] = r.y; w[2] = r.z; w[3] = r.w;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t t = t0 + 2 * j;
+            const int64_t last = n_b > 0 ? n_b - 1 : 0;
+            const uint32_t lo = static_cast<uint16_t>(sc[(t < last ? t : last) * a.stride_n]);
+            const uint32_t hi = static_cast<uint16_t>(sc[(t + 1 < last ? t + 1 : last) * a.stride_n]);
+            w[j] = lo | (hi << 16);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int64_t t = t0 + 2 * j;
+        if (t >= n_b) w[j] |= 0xffffu;
+        if (t + 1 >= n_b) w[j] |= 0xffff0000u;
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__device__ __forceinline__ void unpack_run(const uint4 &r, int (&v)[TK_RUN]) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        v[2 * j] = static_cast<int16_t>(w[j] & 0xffffu);
+        v[2 * j + 1] = static_cast<int16_t>(w[j] >> 16);
+    }
+}
+
+// Lane `tid` owns bins NB-1 - (tid*BPT + j), best scores first, and sums their NG
+// copies; every load of the lane is independent of the others (one round trip).
+template <int NT, int MAX_BPT, int NG>
+__device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, uint32_t (&cnt)[MAX_BPT]) {
+    const int NB = a.n_bins, tid = threadIdx.x;
+    const int BPT = (NB + NT - 1) / NT;
+    const uint32_t *gh = a.hist + static_cast<int64_t>(bh) * NG * NB;
+    uint32_t raw[MAX_BPT][NG];
+#pragma unroll
+    for (int j = 0; j < MAX_BPT; ++j) {
+        const int bi = tid * BPT + j;
+        const bool live = j < BPT && bi < NB;
+        const int bin = live ? NB - 1 - bi : 0;  // unconditional loads, dead bins are dropped below
+#pragma unroll
+        for (int g = 0; g < NG; ++g) raw[j][g] = gh[g * NB + bin];
+    }
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < MAX_BPT; ++j) {
+        const int bi = tid * BPT + j;
+        uint32_t c = 0;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) c += raw[j][g];
+        cnt[j] = (j < BPT && bi < NB) ? c : 0u;
+        mine += cnt[j];
+    }
+    return mine;
+}
+
+// Block-wide search of the threshold bin; every lane returns (thr, need).
+template <int NT, int MAX_BPT>
+__device__ __forceinline__ void find_threshold(const select_args &a, const uint32_t (&cnt)[MAX_BPT],
+                                               uint32_t mine, int k_eff, uint32_t *s_wave, int *s_tn,
+                                               int &thr, int &need) {
+    const int NB = a.n_bins, tid = threadIdx.x;
+    const int BPT = (NB + NT - 1) / NT;
+    if (tid == 0) { s_tn[0] = NB; s_tn[1] = 0; }  // selects nothing unless a lane finds the bin
+    uint32_t total;
+    uint32_t cum = block_exclusive_sum<NT>(mine, s_wave, &total);
+#pragma unroll
+    for (int j = 0; j < MAX_BPT; ++j) {
+        if (k_eff > 0 && cum < static_cast<uint32_t>(k_eff) && cum + cnt[j] >= static_cast<uint32_t>(k_eff)) {
+            s_tn[0] = NB - 1 - (tid * BPT + j);
+            s_tn[1] = k_eff - static_cast<int>(cum);
+        }
+        cum += cnt[j];
+    }
+    __syncthreads();
+    thr = s_tn[0];
+    need = s_tn[1];
+}
+
+__device__ __forceinline__ uint32_t count_run(const uint4 &r, int thr) {
+    int v[TK_RUN];
+    unpack_run(r, v);
+    uint32_t gt = 0, eq = 0;
+#pragma unroll
+    for (int j = 0; j < TK_RUN; ++j) {
+        gt += v[j] > thr;
+        eq += v[j] == thr;
+    }
+    return gt | (eq << 16);
+}
+
+// Places the kept tokens of one block.  (tg, te): tokens above / at the threshold
+// in all earlier blocks.  With LIST the tokens are also written, in order, to the
+// LDS list `s_list` and *n_kept receives their number.  Contains barriers.
+template <int NT, bool LIST = false>
+__device__ __forceinline__ void place_block(const uint4 &run, int64_t t0, int thr, int need, int k_eff,
+                                            uint32_t tg, uint32_t te, uint32_t *s_wave, int32_t *out,
+                                            int32_t *s_list = nullptr, int *n_kept = nullptr) {
+    const uint32_t uneed = static_cast<uint32_t>(need);
+    uint32_t tot;
+    const uint32_t ex = block_exclusive_sum<NT>(count_run(run, thr), s_wave, &tot);
+    int v[TK_RUN];
+    unpack_run(run, v);
+    uint32_t gt_before = tg + (ex & 0xffffu), eq_before = te + (ex >> 16);
+    const uint32_t first = tg + (te < uneed ? te : uneed);  // output position of the block's first kept token
+#pragma unroll
+    for (int j = 0; j < TK_RUN; ++j) {
+        const int s = v[j];
+        if (s > thr) {
+            const uint32_t pos = gt_before + (eq_before < uneed ? eq_before : uneed);
+            if (pos < static_cast<uint32_t>(k_eff)) {
+                out[pos] = static_cast<int32_t>(t0 + j);
+                if constexpr (LIST) s_list[pos - first] = static_cast<int32_t>(t0 + j);
+            }
+            ++gt_before;
+        } else if (s == thr) {
+            if (eq_before < uneed) {
+                const uint32_t pos = gt_before + eq_before;
+                if (pos < static_cast<uint32_t>(k_eff)) {
+                    out[pos] = static_cast<int32_t>(t0 + j);
+                    if constexpr (LIST) s_list[pos - first] = static_cast<int32_t>(t0 + j);
+                }
+            }
+            ++eq_before;
+        }
+    }
+    if constexpr (LIST) {
+        const uint32_t eq_end = te + (tot >> 16);
+        uint32_t end = tg + (tot & 0xffffu) + (eq_end < uneed ? eq_end : uneed);
+        if (end > static_cast<uint32_t>(k_eff)) end = static_cast<uint32_t>(k_eff);
+        *n_kept = end > first ? static_cast<int>(end - first) : 0;
+    }
+}
