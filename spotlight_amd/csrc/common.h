@@ -187,9 +187,9 @@ __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 
 // Exclusive prefix sum of one uint32 per thread over a block of NT threads
-// (NT multiple of 64, <= 1024).  `wave_tot` is NT/64 + 1 words of LDS.
-// Returns the exclusive prefix; *total receives the block sum.  Contains two
-// barriers; every thread of the block must call it.
+// (NT multiple of 64, <= 1024).  `wave_tot` is NT/64 words of LDS that no lane
+// may still be reading from an earlier use.  Returns the exclusive prefix; *total
+// receives the block sum.  One barrier; every thread of the block must call it.
 template <int NT>
 __device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t x, uint32_t *wave_tot,
                                                         uint32_t *total) {
@@ -197,14 +197,28 @@ __device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t x, uint32_t *wa
     const uint32_t inc = wave_inclusive_sum(x);
     if (lane_id() == 63) wave_tot[wave_id()] = inc;
     __syncthreads();
-    if (threadIdx.x < 64) {
-        uint32_t t = threadIdx.x < NW ? wave_tot[threadIdx.x] : 0u;
-        uint32_t ti = wave_inclusive_sum(t);
-        if (threadIdx.x < NW) wave_tot[threadIdx.x] = ti - t;
-        if (threadIdx.x == 63) wave_tot[NW] = ti;
+    uint32_t base = 0, tot = 0;
+    const int w = wave_id();
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+        const uint32_t v = wave_tot[i];
+        tot += v;
+        base += i < w ? v : 0u;
     }
-    __syncthreads();
-    const uint32_t base = wave_tot[wave_id()];
-    *total = wave_tot[NW];
+    *total = tot;
     return base + inc - x;
+}
+
+// Block sums of two values at once (one barrier).  `wave_tot`: 2 * NT/64 words of LDS.
+template <int NT>
+__device__ __forceinline__ void block_sum2(uint32_t a, uint32_t b, uint32_t *wave_tot, uint32_t *ta, uint32_t *tb) {
+    constexpr int NW = NT / 64;
+    const uint32_t ia = wave_inclusive_sum(a), ib = wave_inclusive_sum(b);
+    if (lane_id() == 63) { wave_tot[wave_id()] = ia; wave_tot[NW + wave_id()] = ib; }
+    __syncthreads();
+    uint32_t sa = 0, sb = 0;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) { sa += wave_tot[i]; sb += wave_tot[NW + i]; }
+    *ta = sa;
+    *tb = sb;
 }

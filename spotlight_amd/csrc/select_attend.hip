@@ -50,16 +50,13 @@ __device__ __forceinline__ void sa_select(const select_args &a, int blk, int bh,
         pe += c >> 16;
     }
     uint32_t tg, te;
-    block_exclusive_sum<SA_THREADS>(pg, s_wave, &tg);
-    __syncthreads();
-    block_exclusive_sum<SA_THREADS>(pe, s_wave, &te);
-    __syncthreads();
+    block_sum2<SA_THREADS>(pg, pe, s_wave + 32, &tg, &te);
     place_block<SA_THREADS, true>(v, t0, thr, need, k_eff, tg, te, s_wave, out, s_list, n_kept);
 }
 
 template <typename T, int G, int NG>
 __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args sa, attn_args aa) {
-    __shared__ uint32_t s_wave[SA_THREADS / 64 + 1];
+    __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
     __shared__ int s_tn[2];
     __shared__ int32_t s_list[SA_BLOCK + SA_NW * 4 * SA_U];
     __shared__ attn_shared<G, SA_NW> sh;

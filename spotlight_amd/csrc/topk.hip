@@ -107,10 +107,7 @@ __device__ __forceinline__ void select_fused_body(const select_args &a, int blk,
         pe += c >> 16;
     }
     uint32_t tg, te;
-    block_exclusive_sum<TK_THREADS>(pg, s_wave, &tg);
-    __syncthreads();
-    block_exclusive_sum<TK_THREADS>(pe, s_wave, &te);
-    __syncthreads();
+    block_sum2<TK_THREADS>(pg, pe, s_wave + 32, &tg, &te);
     const uint32_t uneed = static_cast<uint32_t>(need);
     if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
     place_block<TK_THREADS>(v, t0, thr, need, k_eff, tg, te, s_wave, out);
@@ -118,7 +115,7 @@ __device__ __forceinline__ void select_fused_body(const select_args &a, int blk,
 
 template <bool CONTIG, int MAX_BPT, int NG>
 __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a) {
-    __shared__ uint32_t s_wave[TK_THREADS / 64 + 1];
+    __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
     __shared__ int s_tn[2];
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
@@ -140,7 +137,7 @@ __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a)
 
 template <bool CONTIG, int MAX_BPT, int NG>
 __global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a) {
-    __shared__ uint32_t s_wave[TK_THREADS / 64 + 1];
+    __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
     __shared__ int s_tn[2];
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
@@ -167,7 +164,7 @@ __global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a)
 
 template <bool CONTIG>
 __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args a) {
-    __shared__ uint32_t s_wave[TK_THREADS / 64 + 1];
+    __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.KH, h = bh % a.KH;
@@ -191,10 +188,7 @@ __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args 
         pe += c >> 16;
     }
     uint32_t tg, te;
-    block_exclusive_sum<TK_THREADS>(pg, s_wave, &tg);
-    __syncthreads();
-    block_exclusive_sum<TK_THREADS>(pe, s_wave, &te);
-    __syncthreads();
+    block_sum2<TK_THREADS>(pg, pe, s_wave + 32, &tg, &te);
     const uint32_t uneed = static_cast<uint32_t>(need);
     if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
     place_block<TK_THREADS>(v, t0, thr, need, k_eff, tg, te, s_wave, out);
