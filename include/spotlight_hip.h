@@ -233,7 +233,8 @@ typedef struct {
     void *k_res, *v_res;
     int32_t *slots_out;     /* [B, KH, k]                                       */
     uint32_t *lru_stats;    /* [B, KH, 2]                                       */
-    uint32_t *step_counter; /* [1] device counter, incremented every step       */
+    uint32_t *step_counter; /* [1] device counter, incremented every step; needed  */
+                            /* by the LRU and by the one-launch hash + score       */
     /* scratch */
     void *ws;
     size_t ws_bytes;

@@ -147,17 +147,16 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     sl_select_carve(ta, ws + L.select, p.n_cap);
     ha.zero_words = ta.hist;  // the scorer of this step starts from a clean histogram
     ha.zero_count = static_cast<int64_t>(p.B) * p.KH * ta.n_bins * ta.hist_groups;
+    // 2. score seq_lens[b] + 1 rows
+    hamming_args sa{};
+    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.hist_span = ta.hist_span; sa.seq_lens = p.seq_lens;
+    sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
+    sa.n_bins = G * p.nbits + 1; sa.len_bias = 1; sa.n = p.n_max; sa.n_cap = p.n_cap;
+    sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
     if (stages & SL_STAGE_HASH) {
         rc = sl_hash_launch(ha, s);
         if (rc != SL_OK) return rc;
     }
-
-    // 2. score seq_lens[b] + 1 rows
-    hamming_args sa{};
-    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.seq_lens = p.seq_lens;
-    sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
-    sa.n_bins = G * p.nbits + 1; sa.len_bias = 1; sa.n = p.n_max; sa.n_cap = p.n_cap;
-    sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
     if (stages & SL_STAGE_SCORE) {
         rc = sl_hamming_launch(sa, true, s);
         if (rc != SL_OK) return rc;

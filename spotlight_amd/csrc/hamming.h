@@ -12,6 +12,7 @@ struct hamming_args {
     int16_t *out;             // plain: [B, n, KH]; fused: [B, KH, n_cap]
     uint32_t *hist;           // fused: [B, KH, hist_groups, n_bins] global histogram copies
     int hist_groups;
+    int hist_span;            // fused: token t is counted into copy (t / hist_span) % hist_groups
     const int32_t *seq_lens;  // optional per-batch token count
     int B, KH, G, W, head_map;
     int n_bins;               // fused: G*W*32 + 1

@@ -38,7 +38,6 @@ __device__ __forceinline__ void load_code(const uint32_t *p, uint32_t (&c)[W]) {
 template <int W, int G_T, bool FUSED>
 __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     extern __shared__ uint32_t smem[];
-    __shared__ int s_range[2];  // smallest / largest score of this workgroup (fused flavour)
     const int b = blockIdx.y;
     const int KH = a.KH;
     const int G = G_T > 0 ? G_T : a.G;
@@ -61,6 +60,9 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     uint32_t *hist = q_lds + (G_T > 0 ? 0 : KH * G * W);
     const int NB = a.n_bins;
 
+    // the query codes and the HS_U records of the lane are independent loads: all
+    // are issued before the first wait.  Record loads are unconditional (rows past
+    // the end re-read the last row and are discarded below): no branch sits between them
     const uint32_t *qb = a.q_code + static_cast<int64_t>(b) * a.q_stride_b;
     uint32_t qreg[(G_T > 0 ? G_T : 1)][W];
     if constexpr (G_T > 0) {
@@ -69,23 +71,8 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
             const int qh = a.head_map == SL_HEADMAP_BLOCKED ? h * G_T + g : g * KH + h;
             load_code<W>(qb + static_cast<int64_t>(qh) * W, qreg[g]);
         }
-    } else {
-        // q_lds[(h*G + g)*W + w]
-        for (int e = tid; e < KH * G * W; e += HS_THREADS) {
-            const int w = e % W, hg = e / W, g = hg % G, hh = hg / G;
-            const int qh = a.head_map == SL_HEADMAP_BLOCKED ? hh * G + g : g * KH + hh;
-            q_lds[e] = qb[static_cast<int64_t>(qh) * W + w];
-        }
     }
-    if constexpr (FUSED) {
-        for (int e = tid; e < KH * NB; e += HS_THREADS) hist[e] = 0;
-        if (tid == 0) { s_range[0] = NB - 1; s_range[1] = 0; }
-    }
-    if constexpr (FUSED || G_T == 0) __syncthreads();
-
     const uint32_t *kb = a.k_code + static_cast<int64_t>(b) * a.k_stride_b;
-    // loads are unconditional (rows past the end re-read the last row and are
-    // discarded below): no branch sits between the HS_U loads
     uint32_t kreg[HS_U][W];
     bool valid[HS_U];
 #pragma unroll
@@ -95,9 +82,20 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
         const int64_t tc = valid[u] ? t : n_b - 1;
         load_code<W>(kb + (tc * KH + h) * W, kreg[u]);
     }
+    if constexpr (G_T == 0) {
+        // q_lds[(h*G + g)*W + w]
+        for (int e = tid; e < KH * G * W; e += HS_THREADS) {
+            const int w = e % W, hg = e / W, g = hg % G, hh = hg / G;
+            const int qh = a.head_map == SL_HEADMAP_BLOCKED ? hh * G + g : g * KH + hh;
+            q_lds[e] = qb[static_cast<int64_t>(qh) * W + w];
+        }
+    }
+    if constexpr (FUSED) {
+        for (int e = tid; e < KH * NB; e += HS_THREADS) hist[e] = 0;
+    }
+    if constexpr (FUSED || G_T == 0) __syncthreads();
 
     const int full = G * W * 32;
-    int smin = NB - 1, smax = 0;
 #pragma unroll
     for (int u = 0; u < HS_U; ++u) {
         int dist = 0;
@@ -115,11 +113,7 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
         const int score = full - dist;  // matching bits
         const int64_t t = t0 + static_cast<int64_t>(u) * tok_per_pass + tl;
         if constexpr (FUSED) {
-            if (valid[u]) {
-                atomicAdd(&hist[h * NB + score], 1u);
-                smin = score < smin ? score : smin;
-                smax = score > smax ? score : smax;
-            }
+            if (valid[u]) atomicAdd(&hist[h * NB + score], 1u);
             sc_lds[h * (tok_per_pass * HS_U) + u * tok_per_pass + tl] =
                 static_cast<int16_t>(valid[u] ? score : 0);
         } else {
@@ -129,39 +123,32 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     }
 
     if constexpr (FUSED) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            smin = min(smin, __shfl_xor(smin, o, 64));
-            smax = max(smax, __shfl_xor(smax, o, 64));
-        }
-        if ((tid & 63) == 0) {
-            atomicMin(&s_range[0], smin);
-            atomicMax(&s_range[1], smax);
-        }
         __syncthreads();
         // head-major score rows: T int16 per head, four per lane
         const int T = tok_per_pass * HS_U;  // = 1024 / KH, a multiple of 4
-        const int e = tid * 4;
-        const int hh = e / T, tt = e % T;
+        const int e4 = tid * 4;
+        const int hh4 = e4 / T, tt = e4 % T;
         const int64_t t = t0 + tt;
         if (t < a.n_cap) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(sc_lds + e);
-            int16_t *dst = a.out + (static_cast<int64_t>(b) * KH + hh) * a.n_cap + t;
+            const uint2 v = *reinterpret_cast<const uint2 *>(sc_lds + e4);
+            int16_t *dst = a.out + (static_cast<int64_t>(b) * KH + hh4) * a.n_cap + t;
             *reinterpret_cast<uint2 *>(dst) = v;
         }
         // hist_groups copies of the global histogram spread the same-bin adds of the
-        // many workgroups of one (b, kv head) over as many addresses.  Only the
-        // bins between the smallest and largest score seen by this workgroup can
-        // be non-empty, so only those are visited.
-        const int lo = s_range[0], span = s_range[1] - lo + 1;
-        const int grp = blockIdx.x % a.hist_groups;
-        uint32_t *gh = a.hist + (static_cast<int64_t>(b) * KH * a.hist_groups + grp) * NB + lo;
-        for (int hh = 0; hh < KH; ++hh) {
-            const uint32_t *lh = hist + hh * NB + lo;
-            uint32_t *ghh = gh + static_cast<int64_t>(hh) * a.hist_groups * NB;
-            for (int i = tid; i < span; i += HS_THREADS) {
-                const uint32_t c = lh[i];
-                if (c) atomicAdd(&ghh[i], c);
+        // many workgroups of one (b, kv head) over as many addresses; the copy is
+        // picked by token span, which the selector relies on.  Every lane
+        // visits KH*NB/256 bins of the workgroup's table (independent LDS reads) and
+        // adds the non-empty ones; e / NB by multiplication (e * NB < 2^32).
+        const int grp = static_cast<int>(t0 / a.hist_span) % a.hist_groups;
+        uint32_t *gh = a.hist + (static_cast<int64_t>(b) * KH * a.hist_groups + grp) * NB;
+        const uint32_t inv = 0xffffffffu / static_cast<uint32_t>(NB) + 1u;
+        const int total = KH * NB;
+#pragma unroll 4
+        for (int e = tid; e < total; e += HS_THREADS) {
+            const uint32_t c = hist[e];
+            if (c) {
+                const int hh = static_cast<int>(__umulhi(static_cast<uint32_t>(e), inv));
+                atomicAdd(&gh[static_cast<int64_t>(hh) * a.hist_groups * NB + (e - hh * NB)], c);
             }
         }
     }
@@ -226,6 +213,8 @@ __global__ __launch_bounds__(256) void hamming_u8_kernel(const uint8_t *__restri
 }  // namespace
 
 int sl_hamming_launch(const hamming_args &a, bool fused, hipStream_t s) {
+    // a workgroup's tokens must fall into one histogram copy
+    if (fused) SL_REQUIRE(a.hist && a.hist_groups > 0 && a.hist_span > 0 && a.hist_span % (HS_THREADS * HS_U / a.KH) == 0, SL_ERR_SHAPE);
     return fused ? dispatch_w<true>(a, s) : dispatch_w<false>(a, s);
 }
 

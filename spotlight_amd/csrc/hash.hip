@@ -10,6 +10,9 @@
 //                 r, r+RPP, ...; partial sums meet in LDS [RPP][d_hid];
 //   projection 2  [d_hid, 128]: lane (cg2, r2) holds 8 columns of rows
 //                 r2, r2+64, ...; partial sums meet in LDS [64][128];
+//   both LDS tables hold 8192 partial sums and are folded in two steps by all
+//   1024 lanes (8 rows per lane, then one lane per column adds the 1024/columns
+//   sub-totals), so no lane walks a long serial chain of LDS reads;
 //   the 128 pre-activations are turned into sign bits with a wave ballot and
 //   stored as packed words straight into their destination (the query-code
 //   buffer or the cache row of the new key).
@@ -27,6 +30,7 @@ constexpr int HK_THREADS = 1024;
 constexpr int HK_DIN = 128;
 constexpr int HK_NBITS = 128;
 constexpr int HK_B_PER_WG = 4;  // batch rows one workgroup loops over
+constexpr int HK_FOLD = 8;      // rows of a partial-sum table one lane folds in the first step
 
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
@@ -35,15 +39,40 @@ template <int D_HID> struct l1_shape {
     static constexpr int RPP = HK_THREADS / LPR;      // rows per pass
     static constexpr int PASSES = HK_DIN / RPP;       // rows per lane
     static_assert(PASSES >= 1, "d_hid too small for 1024 lanes");
+    static_assert(RPP * D_HID == HK_THREADS * HK_FOLD, "partial-sum table is 8 entries per lane");
 };
 
+// Column sums of the partial-sum table red[ROWS][COLS] (ROWS * COLS = 8192) with
+// all lanes: lane (part, col) adds 8 rows into sub[part][col], then the lanes
+// tid < COLS add the ROWS / 8 sub-totals of their column.  Returns the column sum
+// in lanes tid < COLS (0 elsewhere).  Two barriers; `red` may be rewritten after it.
+template <int COLS>
+__device__ __forceinline__ float fold_columns(const float *red, float *sub) {
+    constexpr int PARTS = HK_THREADS / COLS;
+    const int tid = threadIdx.x;
+    const int col = tid % COLS, part = tid / COLS;
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < HK_FOLD; ++i) s += red[(part * HK_FOLD + i) * COLS + col];
+    sub[part * COLS + col] = s;
+    __syncthreads();
+    float total = 0.f;
+    if (tid < COLS) {
+#pragma unroll
+        for (int i = 0; i < PARTS; ++i) total += sub[i * COLS + tid];
+    }
+    return total;
+}
+
+// One workgroup of HK_THREADS lanes hashes head blockIdx.x (numbered over both
+// sides) for the batch rows [blockIdx.y * HK_B_PER_WG, ..).
 template <typename T, int NL, int D_HID>
 __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     using S1 = l1_shape<D_HID>;
     constexpr int P2 = NL == 2 ? D_HID / 64 : 1;     // second projection: 64 rows per pass
-    constexpr int RED = (S1::RPP * D_HID > 64 * HK_NBITS) ? S1::RPP * D_HID : 64 * HK_NBITS;
     __shared__ float xs[HK_DIN];
-    __shared__ __align__(16) float red[RED];
+    __shared__ __align__(16) float red[HK_THREADS * HK_FOLD];
+    __shared__ float sub[HK_THREADS];
     __shared__ float hidl[D_HID];
 
     const int tid = threadIdx.x;
@@ -51,8 +80,21 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     const int side_i = (a.n_sides > 1 && hh >= a.side[0].H) ? 1 : 0;
     const hash_side &sd = a.side[side_i];
     const int h = hh - (side_i ? a.side[0].H : 0);
+    const int b_lo = blockIdx.y * HK_B_PER_WG;
+    const int b_hi = b_lo + HK_B_PER_WG < a.B ? b_lo + HK_B_PER_WG : a.B;
 
-    // weights -> registers, all loads issued before anything else
+    // every load of the workgroup is issued before anything waits: the inputs of
+    // its batch rows first (they are needed first), then the weights of both
+    // projections, the biases and the K / V rows the launch appends
+    const T *xh = static_cast<const T *>(sd.x) + static_cast<int64_t>(h) * HK_DIN;
+    // (named scalars, picked by the loop counter below: an indexed array would not stay in registers)
+    static_assert(HK_B_PER_WG == 4, "four named input registers");
+    const T *xlane = xh + (tid & (HK_DIN - 1));
+    const int nb = b_hi - b_lo;
+    const float x0 = to_f32(xlane[static_cast<int64_t>(b_lo) * sd.x_stride_b]);
+    const float x1 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 1 ? 1 : 0)) * sd.x_stride_b]);
+    const float x2 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 2 ? 2 : 0)) * sd.x_stride_b]);
+    const float x3 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 3 ? 3 : 0)) * sd.x_stride_b]);
     const int cg = tid % S1::LPR, r = tid / S1::LPR;
     float w1r[S1::PASSES][8];
     {
@@ -67,41 +109,42 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
 #pragma unroll
         for (int q = 0; q < P2; ++q) load8<T>(w2 + static_cast<int64_t>(r2 + 64 * q) * HK_NBITS, w2r[q]);
     }
-    float bias1 = 0.f, bias2 = 0.f;
-    if (sd.b1 && tid < D_HID) bias1 = to_f32(static_cast<const T *>(sd.b1)[static_cast<int64_t>(h) * D_HID + tid]);
-    if (NL == 2 && sd.b2 && tid < HK_NBITS)
-        bias2 = to_f32(static_cast<const T *>(sd.b2)[static_cast<int64_t>(h) * HK_NBITS + tid]);
+    // optional operands are loaded without a branch (an absent one re-reads the
+    // input row and is ignored): a load under a condition would have to be waited
+    // for inside that branch, and with it every load issued before it
+    const T *b1p = sd.b1 ? static_cast<const T *>(sd.b1) + static_cast<int64_t>(h) * D_HID + (tid < D_HID ? tid : 0) : xh;
+    const T *b2p = (NL == 2 && sd.b2) ? static_cast<const T *>(sd.b2) + static_cast<int64_t>(h) * HK_NBITS + (tid & (HK_NBITS - 1)) : xh;
+    const float bias1 = to_f32(*b1p), bias2 = to_f32(*b2p);
+    // appended rows: (b_hi - b_lo) * CH <= 128 chunks of 16 bytes per tensor, one per lane
+    constexpr int CH = HK_DIN * sizeof(T) / 16;
+    const bool cp_live = tid < (b_hi - b_lo) * CH;
+    const int cp_b = b_lo + (cp_live ? tid / CH : 0), cp_c = cp_live ? tid % CH : 0;
+    // destination rows of the batch rows (and of the lane's chunk of the appended rows)
+    const int32_t *rowp = sd.code_row ? sd.code_row : reinterpret_cast<const int32_t *>(sd.codes);
+    const int32_t row0 = rowp[sd.code_row ? b_lo : 0];
+    const int32_t row1 = rowp[sd.code_row ? b_lo + (nb > 1 ? 1 : 0) : 0];
+    const int32_t row2 = rowp[sd.code_row ? b_lo + (nb > 2 ? 2 : 0) : 0];
+    const int32_t row3 = rowp[sd.code_row ? b_lo + (nb > 3 ? 3 : 0) : 0];
+    const int32_t cp_row = rowp[sd.code_row ? cp_b : 0];
+    const T *src0 = sd.copy_src[0] ? static_cast<const T *>(sd.copy_src[0]) : static_cast<const T *>(sd.x);
+    const T *src1 = sd.copy_src[1] ? static_cast<const T *>(sd.copy_src[1]) : static_cast<const T *>(sd.x);
+    const int64_t cp_off = static_cast<int64_t>(cp_b) * sd.x_stride_b + h * HK_DIN;
+    const uint4 cp0 = reinterpret_cast<const uint4 *>(src0 + cp_off)[cp_c];
+    const uint4 cp1 = reinterpret_cast<const uint4 *>(src1 + cp_off)[cp_c];
 
-    // housekeeping that rides along: clear the next score histogram, append K / V rows
+    // housekeeping that rides along: clear the next score histogram
     if (a.zero_words) {
         const int64_t n_wg = static_cast<int64_t>(gridDim.x) * gridDim.y;
-        const int64_t per_wg = (a.zero_count + n_wg - 1) / n_wg;
-        const int64_t z0 = (static_cast<int64_t>(blockIdx.y) * gridDim.x + blockIdx.x) * per_wg;
-        for (int64_t i = z0 + tid; i < z0 + per_wg && i < a.zero_count; i += HK_THREADS) a.zero_words[i] = 0u;
-    }
-    const int b_lo = blockIdx.y * HK_B_PER_WG;
-    const int b_hi = b_lo + HK_B_PER_WG < a.B ? b_lo + HK_B_PER_WG : a.B;
-    {
-        constexpr int CH = HK_DIN * sizeof(T) / 16;  // 16-byte chunks per row
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            if (!sd.copy_src[i]) continue;
-            for (int e = tid; e < (b_hi - b_lo) * CH; e += HK_THREADS) {
-                const int b = b_lo + e / CH, c = e % CH;
-                const uint4 *src = reinterpret_cast<const uint4 *>(
-                    static_cast<const T *>(sd.copy_src[i]) + static_cast<int64_t>(b) * sd.x_stride_b + h * HK_DIN);
-                const int64_t rowi = sd.code_row ? sd.code_row[b] : 0;
-                uint4 *dst = reinterpret_cast<uint4 *>(
-                    static_cast<T *>(sd.copy_dst[i]) + static_cast<int64_t>(b) * sd.copy_dst_stride_b +
-                    rowi * sd.copy_dst_stride_n + h * HK_DIN);
-                dst[c] = src[c];
-            }
-        }
+        const int64_t wg = static_cast<int64_t>(blockIdx.y) * gridDim.x + blockIdx.x;
+        for (int64_t i = wg * HK_THREADS + tid; i < a.zero_count; i += n_wg * HK_THREADS) a.zero_words[i] = 0u;
     }
 
-    const T *xh = static_cast<const T *>(sd.x) + static_cast<int64_t>(h) * HK_DIN;
+#pragma unroll 1  // keeps the kernel small: it mostly runs on compute units that do not hold its code yet
     for (int b = b_lo; b < b_hi; ++b) {
-        if (tid < HK_DIN) xs[tid] = to_f32(xh[static_cast<int64_t>(b) * sd.x_stride_b + tid]);
+        const int bi = b - b_lo;
+        const float x_cur = bi == 0 ? x0 : bi == 1 ? x1 : bi == 2 ? x2 : x3;
+        const int32_t row_b = bi == 0 ? row0 : bi == 1 ? row1 : bi == 2 ? row2 : row3;
+        if (tid < HK_DIN) xs[tid] = x_cur;
         __syncthreads();
 
         // first projection
@@ -118,12 +161,9 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
             dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
         }
         __syncthreads();
-        float v1 = 0.f;
+        float v1 = fold_columns<D_HID>(red, sub);
         if (tid < D_HID) {
-            float sum = 0.f;
-#pragma unroll 8
-            for (int rr = 0; rr < S1::RPP; ++rr) sum += red[rr * D_HID + tid];
-            v1 = round_to<T>(sum);
+            v1 = round_to<T>(v1);
             if (sd.b1) v1 = round_to<T>(v1 + bias1);
             if constexpr (NL == 2) {
                 v1 = round_to<T>(silu_f32(v1));
@@ -134,7 +174,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
             }
         }
         uint32_t *code_dst = sd.codes + static_cast<int64_t>(b) * sd.code_stride_b +
-                             static_cast<int64_t>(sd.code_row ? sd.code_row[b] : 0) * sd.code_stride_n +
+                             static_cast<int64_t>(sd.code_row ? row_b : 0) * sd.code_stride_n +
                              static_cast<int64_t>(h) * sd.code_stride_h;
         if constexpr (NL == 1) {
             // waves 0 .. D_HID/64-1 hold the pre-activations: 64 sign bits per wave
@@ -160,12 +200,9 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
                 dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
             }
             __syncthreads();
-            float v2 = 0.f;
+            float v2 = fold_columns<HK_NBITS>(red, sub);
             if (tid < HK_NBITS) {
-                float sum = 0.f;
-#pragma unroll 8
-                for (int rr = 0; rr < 64; ++rr) sum += red[rr * HK_NBITS + tid];
-                v2 = round_to<T>(sum);
+                v2 = round_to<T>(v2);
                 if (sd.b2) v2 = round_to<T>(v2 + bias2);
                 if (a.residue) v2 = round_to<T>(v2 + hidl[tid]);
             }
@@ -176,6 +213,14 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
             }
             __syncthreads();
         }
+    }
+
+    // cache append of the new K and V rows (loaded at the top)
+    if (cp_live) {
+        const int64_t dst_off = static_cast<int64_t>(cp_b) * sd.copy_dst_stride_b +
+                                static_cast<int64_t>(sd.code_row ? cp_row : 0) * sd.copy_dst_stride_n + h * HK_DIN;
+        if (sd.copy_src[0]) reinterpret_cast<uint4 *>(static_cast<T *>(sd.copy_dst[0]) + dst_off)[cp_c] = cp0;
+        if (sd.copy_src[1]) reinterpret_cast<uint4 *>(static_cast<T *>(sd.copy_dst[1]) + dst_off)[cp_c] = cp1;
     }
 }
 

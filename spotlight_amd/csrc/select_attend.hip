@@ -2,8 +2,9 @@
 // in one launch.
 //
 // One workgroup of 8 waves per 4096-token block of a (b, kv head).  It derives
-// (thr, need) from the histogram, counts the blocks before its own, places its
-// kept tokens -- into the global index list AND into an LDS list -- and then
+// (thr, need) from the histogram, takes the number of kept tokens in front of
+// its block from the histogram copies of the earlier blocks, places its kept
+// tokens into an LDS list (copied out to the global index list) and then
 // attends over exactly those rows (attn_core.h), as run `block` of the
 // (b, kv head).  Compared with select + attention as two launches this removes
 // one launch and the store -> load round trip of the index list; the runs are
@@ -20,39 +21,12 @@ namespace {
 constexpr int SA_NW = 8;
 constexpr int SA_THREADS = SA_NW * 64;
 constexpr int SA_BLOCK = SA_THREADS * TK_RUN;   // 4096 tokens
-constexpr int SA_U = 2;                         // row groups in flight per iteration (64 rows per workgroup)
+constexpr int SA_U = 4;                         // row groups in flight per iteration (128 rows per workgroup)
 constexpr int SA_MAX_BPT = 2;                   // histogram bins per lane (<= 1024 bins)
 
 template <bool dummy = true> struct sa_static_checks {
     static_assert(SA_MAX_BLOCKS == AT_MAX_SPLITS, "one attention run per token block");
 };
-
-template <int NG, int NPREV>
-__device__ __forceinline__ void sa_select(const select_args &a, int blk, int bh, int b, int h, int64_t n_b, int k_eff,
-                                          int32_t *out, uint32_t *s_wave, int *s_tn, int32_t *s_list, int *n_kept) {
-    const int tid = threadIdx.x;
-    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
-    const int64_t t0 = static_cast<int64_t>(blk) * SA_BLOCK + tid * TK_RUN;
-    const uint4 v = load_run<true>(a, sc, t0, n_b);
-    uint4 prev[NPREV > 0 ? NPREV : 1];
-#pragma unroll
-    for (int j = 0; j < NPREV; ++j)
-        prev[j] = load_run<true>(a, sc, static_cast<int64_t>(j < blk ? j : blk) * SA_BLOCK + tid * TK_RUN, n_b);
-    uint32_t cnt[SA_MAX_BPT];
-    const uint32_t mine = load_bins<SA_THREADS, SA_MAX_BPT, NG>(a, bh, cnt);
-    int thr, need;
-    find_threshold<SA_THREADS, SA_MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
-    uint32_t pg = 0, pe = 0;
-#pragma unroll
-    for (int j = 0; j < NPREV; ++j) {
-        const uint32_t c = j < blk ? count_run(prev[j], thr) : 0u;
-        pg += c & 0xffffu;
-        pe += c >> 16;
-    }
-    uint32_t tg, te;
-    block_sum2<SA_THREADS>(pg, pe, s_wave + 32, &tg, &te);
-    place_block<SA_THREADS, true>(v, t0, thr, need, k_eff, tg, te, s_wave, out, s_list, n_kept);
-}
 
 template <typename T, int G, int NG>
 __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args sa, attn_args aa) {
@@ -64,6 +38,14 @@ __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args s
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int bh = b * sa.KH + h;
+    // loads first: none of them needs the sequence length.  One histogram copy per
+    // token block, so the copies in front of this block count the tokens in front of it.
+    const int16_t *sc = sa.score + static_cast<int64_t>(b) * sa.stride_b + static_cast<int64_t>(h) * sa.stride_h;
+    const int64_t t0 = static_cast<int64_t>(blk) * SA_BLOCK + tid * TK_RUN;
+    const uint4 raw = load_run_raw<true>(sa, sc, t0);
+    uint32_t cnt[SA_MAX_BPT], before[SA_MAX_BPT];
+    const uint32_t mine = load_bins<SA_THREADS, SA_MAX_BPT, NG>(sa, bh, blk, cnt, before);
+
     const int64_t n_b = tokens_of(sa, b);
     const int k_eff = n_b < sa.k ? static_cast<int>(n_b) : sa.k;
     int32_t *out = sa.idx + static_cast<int64_t>(bh) * sa.k;
@@ -71,18 +53,22 @@ __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args s
         for (int i = k_eff + tid; i < sa.k; i += SA_THREADS) out[i] = -1;
     if (static_cast<int64_t>(blk) * SA_BLOCK >= n_b) return;
     const int S = static_cast<int>((n_b + SA_BLOCK - 1) / SA_BLOCK);  // runs of this (b, kv head)
+    const uint4 v = mask_run(raw, t0, n_b);
 
-    int n_kept = 0;
-    if (blk == 0) sa_select<NG, 0>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
-    else if (blk <= 1) sa_select<NG, 1>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
-    else if (blk <= 3) sa_select<NG, 3>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
-    else if (blk <= 7) sa_select<NG, 7>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
-    else sa_select<NG, SA_MAX_BLOCKS - 1>(sa, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn, s_list, &n_kept);
+    int thr, need;
+    find_threshold<SA_THREADS, SA_MAX_BPT>(sa, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+    uint32_t pg, pe, tg, te;
+    before_counts<SA_THREADS, SA_MAX_BPT>(sa, before, thr, pg, pe);
+    block_sum2<SA_THREADS>(pg, pe, s_wave + 32, &tg, &te);
+    int n_kept = 0, first = 0;
+    place_block<SA_THREADS, true>(v, t0, thr, need, k_eff, tg, te, s_wave, out, s_list, &n_kept, &first);
 
-    // pad the list to whole iterations of the attention loop, then attend over it
+    // the list goes out with coalesced stores and is padded to whole iterations of
+    // the attention loop, which then runs over it
     constexpr int ITER = SA_NW * 4 * SA_U;
     const int padded = (n_kept + ITER - 1) / ITER * ITER;
     __syncthreads();
+    for (int i = tid; i < n_kept; i += SA_THREADS) out[first + i] = s_list[i];
     for (int i = n_kept + tid; i < padded; i += SA_THREADS) s_list[i] = -1;
     __syncthreads();
     attend_rows_and_merge<T, G, SA_NW, SA_U>(aa, b, h, blk, S, s_list, n_kept, sh);
@@ -110,7 +96,8 @@ int launch_g(const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t 
 bool sl_select_attend_supported(const select_args &sa, const attn_args &aa) {
     const int G = aa.QH / aa.KH;
     const int64_t blocks = (sa.n + SA_BLOCK - 1) / SA_BLOCK;
-    return (G == 1 || G == 2 || G == 4) && blocks <= SA_MAX_BLOCKS && sa.n_bins <= SA_THREADS * SA_MAX_BPT &&
+    return (G == 1 || G == 2 || G == 4) && blocks <= SA_MAX_BLOCKS && blocks <= sa.hist_groups &&
+           sa.hist_span == SA_BLOCK && sa.n_bins <= SA_THREADS * SA_MAX_BPT &&
            (sa.hist_groups == 4 || sa.hist_groups == 16) && sa.stride_n == 1 && sa.stride_b % 8 == 0 &&
            sa.stride_h % 8 == 0 && sa.stride_h >= (sa.n + 7) / 8 * 8 && sl_aligned(sa.score, 16) && aa.B <= 65535;
 }

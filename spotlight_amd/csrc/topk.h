@@ -9,6 +9,7 @@ struct select_args {
     const int16_t *score;     // element (b, t, h) at b*stride_b + t*stride_n + h*stride_h
     uint32_t *hist;           // [B, KH, hist_groups, n_bins]: the copies are summed
     int hist_groups;          // 4 or 16
+    int hist_span;            // token t is counted into copy (t / hist_span) % hist_groups
     int32_t *thr_need;        // [B, KH, 2] scratch: threshold bin, tokens to take from it
     uint32_t *block_cnt;      // [B, KH, n_blocks] scratch: (above | equal << 16) per token block
     int n_blocks;             // row length of block_cnt
@@ -20,6 +21,7 @@ struct select_args {
 };
 
 int sl_select_hist_groups(int64_t n);
+int64_t sl_select_hist_span(int64_t n);
 size_t sl_select_ws_bytes(int B, int KH, int n_bins, int64_t n);
 // points hist / thr_need / block_cnt of `a` into `ws` (a.B, a.KH, a.n_bins set)
 void sl_select_carve(select_args &a, void *ws, int64_t n_for_blocks);

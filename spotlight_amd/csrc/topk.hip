@@ -21,11 +21,14 @@
 // workgroup derives (thr, need) itself (the histogram is 2 KB).  What it also
 // needs is the number of tokens above / at the threshold in the blocks before
 // its own:
-//   * up to TK_FUSE_BLOCKS blocks, it simply counts them itself -- all those
-//     score loads are issued together with its own, one memory round trip,
-//     one launch (select_fused_kernel);
-//   * beyond that, a first launch writes per-block counts and a second one
-//     sums them (select_count_kernel + select_compact_kernel).
+//   * the histogram is kept as hist_groups copies and the tokens
+//     [c*hist_span, (c+1)*hist_span) are counted into copy c (modulo the number
+//     of copies).  While the cache fits hist_groups*hist_span tokens, the copies
+//     in front of a block ARE the histogram of the tokens in front of it, so the
+//     two numbers fall out of the loads every workgroup does anyway: one launch
+//     (select_fused_kernel), no second pass over earlier scores;
+//   * beyond that the copies wrap around; a first launch writes per-block counts
+//     and a second one sums them (select_count_kernel + select_compact_kernel).
 #include "topk_core.h"
 
 #include <string.h>
@@ -34,7 +37,6 @@ namespace {
 
 constexpr int TK_BLOCK = TK_THREADS * TK_RUN;      // tokens per workgroup
 constexpr int TK_MAX_BPT = (TK_MAX_BINS + TK_THREADS - 1) / TK_THREADS;  // histogram bins a lane owns
-constexpr int TK_FUSE_BLOCKS = 16;                 // single-launch path up to this many blocks (and <= 1024 bins)
 
 __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *p, int64_t n) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, i
         atomicAdd(&hist[h * NB + s], 1u);
     }
     __syncthreads();
-    const int grp = blockIdx.x % a.hist_groups;
+    const int grp = static_cast<int>(t0 / a.hist_span) % a.hist_groups;
     for (int i = threadIdx.x; i < KHg * NB; i += SH_THREADS) {
         const uint32_t c = hist[i];
         const int h = i / NB, bin = i % NB;
@@ -78,40 +80,7 @@ __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, i
     }
 }
 
-// ---- single launch: every block counts the blocks before it ---------------------
-
-// Body for a block with at most NPREV blocks before it: the NPREV loads are
-// unconditional (slots beyond `blk` re-read the own block and are not counted).
-template <bool CONTIG, int MAX_BPT, int NG, int NPREV>
-__device__ __forceinline__ void select_fused_body(const select_args &a, int blk, int bh, int b, int h, int64_t n_b,
-                                                  int k_eff, int32_t *out, uint32_t *s_wave, int *s_tn) {
-    const int tid = threadIdx.x;
-    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
-    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
-    const uint4 v = load_run<CONTIG>(a, sc, t0, n_b);
-    uint4 prev[NPREV > 0 ? NPREV : 1];
-#pragma unroll
-    for (int j = 0; j < NPREV; ++j)
-        prev[j] = load_run<CONTIG>(a, sc, static_cast<int64_t>(j < blk ? j : blk) * TK_BLOCK + tid * TK_RUN, n_b);
-    uint32_t cnt[MAX_BPT];
-    const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, cnt);
-
-    int thr, need;
-    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
-
-    uint32_t pg = 0, pe = 0;
-#pragma unroll
-    for (int j = 0; j < NPREV; ++j) {
-        const uint32_t c = j < blk ? count_run(prev[j], thr) : 0u;
-        pg += c & 0xffffu;
-        pe += c >> 16;
-    }
-    uint32_t tg, te;
-    block_sum2<TK_THREADS>(pg, pe, s_wave + 32, &tg, &te);
-    const uint32_t uneed = static_cast<uint32_t>(need);
-    if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
-    place_block<TK_THREADS>(v, t0, thr, need, k_eff, tg, te, s_wave, out);
-}
+// ---- single launch: the histogram copies in front of a block give its offsets ------
 
 template <bool CONTIG, int MAX_BPT, int NG>
 __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a) {
@@ -120,17 +89,29 @@ __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a)
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.KH, h = bh % a.KH;
+    // loads first: none of them needs the sequence length
+    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
+    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
+    const uint4 raw = load_run_raw<CONTIG>(a, sc, t0);
+    uint32_t cnt[MAX_BPT], before[MAX_BPT];
+    const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, blk * (TK_BLOCK / a.hist_span), cnt, before);
+
     const int64_t n_b = tokens_of(a, b);
     const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
     int32_t *out = a.idx + static_cast<int64_t>(bh) * a.k;
     if (blk == 0)
         for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;
     if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b) return;
-    if (blk == 0) select_fused_body<CONTIG, MAX_BPT, NG, 0>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
-    else if (blk <= 1) select_fused_body<CONTIG, MAX_BPT, NG, 1>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
-    else if (blk <= 3) select_fused_body<CONTIG, MAX_BPT, NG, 3>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
-    else if (blk <= 7) select_fused_body<CONTIG, MAX_BPT, NG, 7>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
-    else select_fused_body<CONTIG, MAX_BPT, NG, TK_FUSE_BLOCKS - 1>(a, blk, bh, b, h, n_b, k_eff, out, s_wave, s_tn);
+    const uint4 v = mask_run(raw, t0, n_b);
+
+    int thr, need;
+    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+    uint32_t pg, pe, tg, te;
+    before_counts<TK_THREADS, MAX_BPT>(a, before, thr, pg, pe);
+    block_sum2<TK_THREADS>(pg, pe, s_wave + 32, &tg, &te);
+    const uint32_t uneed = static_cast<uint32_t>(need);
+    if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
+    place_block<TK_THREADS>(v, t0, thr, need, k_eff, tg, te, s_wave, out);
 }
 
 // ---- two launches: per-block counts, then placement --------------------------------
@@ -142,15 +123,15 @@ __global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a)
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.KH, h = bh % a.KH;
+    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
+    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
+    const uint4 raw = load_run_raw<CONTIG>(a, sc, t0);
+    uint32_t cnt[MAX_BPT], before[MAX_BPT];
+    const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, 0, cnt, before);
     const int64_t n_b = tokens_of(a, b);
     if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b && blk > 0) return;
     const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
-
-    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
-    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
-    const uint4 v = load_run<CONTIG>(a, sc, t0, n_b);
-    uint32_t cnt[MAX_BPT];
-    const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, cnt);
+    const uint4 v = mask_run(raw, t0, n_b);
     int thr, need;
     find_threshold<TK_THREADS, MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
     if (blk == 0 && tid == 0) {
@@ -168,6 +149,9 @@ __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args 
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.KH, h = bh % a.KH;
+    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
+    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
+    const uint4 raw = load_run_raw<CONTIG>(a, sc, t0);
     const int64_t n_b = tokens_of(a, b);
     const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
     int32_t *out = a.idx + static_cast<int64_t>(bh) * a.k;
@@ -175,10 +159,7 @@ __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args 
         for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;
     if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b) return;
     const int thr = a.thr_need[bh * 2], need = a.thr_need[bh * 2 + 1];
-
-    const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
-    const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
-    const uint4 v = load_run<CONTIG>(a, sc, t0, n_b);
+    const uint4 v = mask_run(raw, t0, n_b);
 
     const uint32_t *bc = a.block_cnt + static_cast<int64_t>(bh) * a.n_blocks;
     uint32_t pg = 0, pe = 0;
@@ -205,11 +186,18 @@ int sl_select_tune(const char *key, int value) {
 
 int sl_select_hist_groups(int64_t n) {
     if (g_hist_copies) return g_hist_copies;
-    // Copies of every histogram bin, so that the same-bin adds of the many scorer
-    // workgroups of one (b, kv head) spread over as many addresses: 16 for long
-    // caches, 4 for short ones (fewer workgroups, and the copies must be cleared
-    // and read every step).
-    return n > 20000 ? 16 : 4;
+    // Copies of every histogram bin: they spread the same-bin adds of the many
+    // scorer workgroups of one (b, kv head) over as many addresses, and copy c
+    // counts the tokens of span c, which is what lets one launch select (see the
+    // top of this file).  16 for long caches, 4 for short ones (the copies must be
+    // cleared and read every step).
+    return n > 4 * 4096 ? 16 : 4;
+}
+
+int64_t sl_select_hist_span(int64_t n) {
+    // tokens per copy: 4096 (the block of the fused select + attend kernel) while
+    // 16 of them cover the cache, else this file's block
+    return n > 16 * 4096 ? TK_BLOCK : 4096;
 }
 
 size_t sl_select_ws_bytes(int B, int KH, int n_bins, int64_t n) {
@@ -225,6 +213,7 @@ void sl_select_carve(select_args &a, void *ws, int64_t n_for_blocks) {
     char *p = static_cast<char *>(ws);
     a.hist = reinterpret_cast<uint32_t *>(p);
     a.hist_groups = sl_select_hist_groups(n_for_blocks);
+    a.hist_span = static_cast<int>(sl_select_hist_span(n_for_blocks));
     p += sl_align_up(sizeof(uint32_t) * bh * a.n_bins * a.hist_groups, 256);
     a.thr_need = reinterpret_cast<int32_t *>(p);
     p += sl_align_up(sizeof(int32_t) * bh * 2, 256);
@@ -246,9 +235,12 @@ int sl_select_launch(const select_args &a, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(bh));
     const bool small = a.n_bins <= TK_THREADS;  // one bin per lane: the common case (G * nbits <= 1023)
     SL_REQUIRE(a.hist_groups == 4 || a.hist_groups == 16, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(a.hist_span > 0 && TK_BLOCK % a.hist_span == 0, SL_ERR_UNSUPPORTED);
+    // one launch while the copies do not wrap around (and one bin per lane, contiguous scores)
+    const bool ordered = a.n <= static_cast<int64_t>(a.hist_groups) * a.hist_span;
 #define SL_SELECT_LAUNCH(CONTIG, BPT, NG)                                                        \
     do {                                                                                         \
-        if (CONTIG && BPT == 1 && blocks <= TK_FUSE_BLOCKS) { /* strided scores: two launches */ \
+        if (CONTIG && BPT == 1 && ordered) { /* strided scores: two launches */                  \
             select_fused_kernel<true, 1, NG><<<grid, dim3(TK_THREADS), 0, s>>>(a);               \
         } else {                                                                                 \
             select_count_kernel<CONTIG, BPT, NG><<<grid, dim3(TK_THREADS), 0, s>>>(a);           \

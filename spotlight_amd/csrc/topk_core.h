@@ -18,26 +18,33 @@ __device__ __forceinline__ int64_t tokens_of(const select_args &a, int b) {
 // ---- pieces shared by the select kernels ---------------------------------------
 
 // Eight consecutive scores of one lane as four packed words (token 2j in the low
-// half of word j).  The load is unconditional and branch free: CONTIG reads the
-// 16 bytes at t0 (callers guarantee they lie inside the allocation), the strided
-// flavour clamps each token index; tokens at or beyond n_b then become -1, which
-// never qualifies.
+// half of word j).  load_run_raw is unconditional, branch free and independent of
+// the sequence length, so it can be issued before that length is known: CONTIG
+// reads 16 bytes at t0, moved back to the last run that lies inside the row of
+// a.n tokens (rows are padded to whole runs); the strided flavour clamps each
+// token index.  mask_run then turns tokens at or beyond n_b into -1, which never
+// qualifies (a clamped run only holds such tokens).
 template <bool CONTIG>
-__device__ __forceinline__ uint4 load_run(const select_args &a, const int16_t *sc, int64_t t0, int64_t n_b) {
-    uint32_t w[4];
+__device__ __forceinline__ uint4 load_run_raw(const select_args &a, const int16_t *sc, int64_t t0) {
     if constexpr (CONTIG) {
-        const uint4 r = *reinterpret_cast<const uint4 *>(sc + t0);
-        w[0] = r.x; w[1] = r.y; w[2] = r.z; w[3] = r.w;
+        const int64_t last_run = a.n > TK_RUN ? (a.n - 1) / TK_RUN * TK_RUN : 0;
+        return *reinterpret_cast<const uint4 *>(sc + (t0 < last_run ? t0 : last_run));
     } else {
+        uint32_t w[4];
+        const int64_t last = a.n > 0 ? a.n - 1 : 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int64_t t = t0 + 2 * j;
-            const int64_t last = n_b > 0 ? n_b - 1 : 0;
             const uint32_t lo = static_cast<uint16_t>(sc[(t < last ? t : last) * a.stride_n]);
             const uint32_t hi = static_cast<uint16_t>(sc[(t + 1 < last ? t + 1 : last) * a.stride_n]);
             w[j] = lo | (hi << 16);
         }
+        return make_uint4(w[0], w[1], w[2], w[3]);
     }
+}
+
+__device__ __forceinline__ uint4 mask_run(const uint4 &r, int64_t t0, int64_t n_b) {
+    uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int64_t t = t0 + 2 * j;
@@ -58,8 +65,12 @@ __device__ __forceinline__ void unpack_run(const uint4 &r, int (&v)[TK_RUN]) {
 
 // Lane `tid` owns bins NB-1 - (tid*BPT + j), best scores first, and sums their NG
 // copies; every load of the lane is independent of the others (one round trip).
+// Copy c holds the tokens [c*span, (c+1)*span) (modulo NG), so the sum over the
+// first `copies_before` copies -- returned in `before` -- is the histogram of all
+// tokens in front of a block that starts at copies_before*span.
 template <int NT, int MAX_BPT, int NG>
-__device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, uint32_t (&cnt)[MAX_BPT]) {
+__device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, int copies_before,
+                                              uint32_t (&cnt)[MAX_BPT], uint32_t (&before)[MAX_BPT]) {
     const int NB = a.n_bins, tid = threadIdx.x;
     const int BPT = (NB + NT - 1) / NT;
     const uint32_t *gh = a.hist + static_cast<int64_t>(bh) * NG * NB;
@@ -76,13 +87,35 @@ __device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, uint
 #pragma unroll
     for (int j = 0; j < MAX_BPT; ++j) {
         const int bi = tid * BPT + j;
-        uint32_t c = 0;
+        const bool live = j < BPT && bi < NB;
+        uint32_t c = 0, bf = 0;
 #pragma unroll
-        for (int g = 0; g < NG; ++g) c += raw[j][g];
-        cnt[j] = (j < BPT && bi < NB) ? c : 0u;
+        for (int g = 0; g < NG; ++g) {
+            c += raw[j][g];
+            bf += g < copies_before ? raw[j][g] : 0u;
+        }
+        cnt[j] = live ? c : 0u;
+        before[j] = live ? bf : 0u;
         mine += cnt[j];
     }
     return mine;
+}
+
+// Tokens above / at the threshold in front of the block, from the `before` sums of
+// load_bins: per-lane contributions, to be added up over the workgroup.
+template <int NT, int MAX_BPT>
+__device__ __forceinline__ void before_counts(const select_args &a, const uint32_t (&before)[MAX_BPT], int thr,
+                                              uint32_t &above, uint32_t &equal) {
+    const int NB = a.n_bins, tid = threadIdx.x;
+    const int BPT = (NB + NT - 1) / NT;
+    above = 0;
+    equal = 0;
+#pragma unroll
+    for (int j = 0; j < MAX_BPT; ++j) {
+        const int bin = NB - 1 - (tid * BPT + j);
+        above += bin > thr ? before[j] : 0u;
+        equal += bin == thr ? before[j] : 0u;
+    }
 }
 
 // Block-wide search of the threshold bin; every lane returns (thr, need).
@@ -121,12 +154,14 @@ __device__ __forceinline__ uint32_t count_run(const uint4 &r, int thr) {
 }
 
 // Places the kept tokens of one block.  (tg, te): tokens above / at the threshold
-// in all earlier blocks.  With LIST the tokens are also written, in order, to the
-// LDS list `s_list` and *n_kept receives their number.  Contains barriers.
+// in all earlier blocks.  Without LIST the tokens go to their positions in `out`;
+// with LIST they are written, in order, to the LDS list `s_list` instead, *n_kept
+// receives their number and *first their position in `out` (the caller copies the
+// list out with coalesced stores).  Contains barriers.
 template <int NT, bool LIST = false>
 __device__ __forceinline__ void place_block(const uint4 &run, int64_t t0, int thr, int need, int k_eff,
                                             uint32_t tg, uint32_t te, uint32_t *s_wave, int32_t *out,
-                                            int32_t *s_list = nullptr, int *n_kept = nullptr) {
+                                            int32_t *s_list = nullptr, int *n_kept = nullptr, int *first_pos = nullptr) {
     const uint32_t uneed = static_cast<uint32_t>(need);
     uint32_t tot;
     const uint32_t ex = block_exclusive_sum<NT>(count_run(run, thr), s_wave, &tot);
@@ -137,28 +172,20 @@ __device__ __forceinline__ void place_block(const uint4 &run, int64_t t0, int th
 #pragma unroll
     for (int j = 0; j < TK_RUN; ++j) {
         const int s = v[j];
-        if (s > thr) {
-            const uint32_t pos = gt_before + (eq_before < uneed ? eq_before : uneed);
-            if (pos < static_cast<uint32_t>(k_eff)) {
-                out[pos] = static_cast<int32_t>(t0 + j);
-                if constexpr (LIST) s_list[pos - first] = static_cast<int32_t>(t0 + j);
-            }
-            ++gt_before;
-        } else if (s == thr) {
-            if (eq_before < uneed) {
-                const uint32_t pos = gt_before + eq_before;
-                if (pos < static_cast<uint32_t>(k_eff)) {
-                    out[pos] = static_cast<int32_t>(t0 + j);
-                    if constexpr (LIST) s_list[pos - first] = static_cast<int32_t>(t0 + j);
-                }
-            }
-            ++eq_before;
+        const bool above = s > thr, equal = s == thr;
+        const uint32_t pos = gt_before + (eq_before < uneed ? eq_before : uneed);
+        if ((above || (equal && eq_before < uneed)) && pos < static_cast<uint32_t>(k_eff)) {
+            if constexpr (LIST) s_list[pos - first] = static_cast<int32_t>(t0 + j);
+            else out[pos] = static_cast<int32_t>(t0 + j);
         }
+        gt_before += above;
+        eq_before += equal;
     }
     if constexpr (LIST) {
         const uint32_t eq_end = te + (tot >> 16);
         uint32_t end = tg + (tot & 0xffffu) + (eq_end < uneed ? eq_end : uneed);
         if (end > static_cast<uint32_t>(k_eff)) end = static_cast<uint32_t>(k_eff);
         *n_kept = end > first ? static_cast<int>(end - first) : 0;
+        *first_pos = static_cast<int>(first);
     }
 }
