@@ -14,8 +14,7 @@ namespace {
 
 constexpr int AT_NW = 4;             // waves per workgroup
 constexpr int AT_THREADS = AT_NW * 64;
-constexpr int AT_U = 4;              // row groups in flight per iteration (64 rows per workgroup)
-constexpr int AT_ITER_ROWS = AT_NW * 4 * AT_U;
+constexpr int AT_ITER_ROWS = 64;     // runs are cut at multiples of this many rows
 constexpr int AT_MAX_ROWS = 1024;    // rows per run (LDS row-number buffer)
 // The arrival tickets sit in a fixed-size head of the workspace so that the
 // partials of a call with other shapes can never land on them: the tickets are
@@ -32,7 +31,7 @@ __global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
     const int32_t *idx = a.idx + (static_cast<int64_t>(b) * a.KH + h) * a.k;
     for (int i = threadIdx.x; i < a.rows; i += AT_THREADS) s_row[i] = r_lo + i < r_hi ? idx[r_lo + i] : -1;
     __syncthreads();
-    attend_rows_and_merge<T, G, AT_NW, AT_U>(a, b, h, split, gridDim.x, s_row, a.rows, sh);
+    attend_rows_and_merge<T, G, AT_NW>(a, b, h, split, gridDim.x, s_row, a.rows, sh);
 }
 
 template <typename T, int G>

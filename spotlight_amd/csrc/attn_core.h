@@ -1,20 +1,31 @@
 // Device-side body of the sparse GQA decode attention, shared by the stand-alone
 // attention kernel and the fused select + attend kernel.
 //
-//   * a K or V row of 128 elements is read by 16 lanes with one 16-byte load
-//     each (two for fp32), so a wave covers 4 rows per load; U such row groups
-//     -- K and V alike, V addresses do not depend on the scores -- are in
-//     flight before the first dot product;
-//   * each 16-lane group keeps its 8-element slice of the G query rows in
-//     registers and carries its own running softmax state (max, sum, 8
-//     accumulators per query head), so the G heads of the group reuse every
-//     K/V byte from registers and there is no barrier inside the row loop;
-//   * the lane-group states meet in LDS: one weight exp(m - M) per (group,
-//     head), then every output element is a weighted sum over the groups;
-//   * a run's (acc, max, sum) goes to the workspace through device-coherent
-//     stores; the last workgroup of a (b, kv head) to arrive loads all runs'
-//     partials at once (one round trip) and merges them the same way, in run
-//     order, so the result does not depend on arrival order.
+// The kernels that use it run one or two waves per SIMD, so what they pay for is
+// the number of instructions each wave issues, not bandwidth.  The rows of a run
+// are therefore processed in chunks, and a chunk in two differently laid out
+// phases, each of which does its arithmetic once instead of once per lane:
+//
+//   scores   a K row of 128 elements is read by 16 lanes with one 16-byte load
+//            each.  Every lane forms the partial dot products of its 8-element
+//            slice for 16 (query head, row) pairs -- packed dot2 for 16-bit
+//            inputs -- and a butterfly over the 16 lanes that halves the number
+//            of live values at every step leaves each lane with ONE complete
+//            score, after 15 cross-lane adds instead of 64.  That lane alone
+//            scales it, takes part in the maximum and evaluates the one exp();
+//            the probabilities go to LDS as p[row][head].
+//   values   wave w takes the rows w, w + NW, ... of the chunk; its 64 lanes own
+//            two output columns each, so a V row is one coalesced 256-byte load
+//            and the G accumulators per column stay in registers:
+//            8 FMAs per row for G = 4.  The V loads do not depend on the scores
+//            and are issued together with the K loads.
+//
+// All waves share one running maximum per head, so the per-wave accumulators
+// are simply added in LDS at the end (NW partial tiles, not one per 16 lanes).
+// A run's (acc, max, sum) then goes to the workspace through device-coherent
+// stores; the last workgroup of a (b, kv head) to arrive loads all runs'
+// partials at once (one round trip) and merges them in run order, so the
+// result does not depend on arrival order.
 #pragma once
 #include "attn.h"
 
@@ -22,133 +33,288 @@ constexpr int AT_D = 128;
 constexpr int AT_PART = AT_D + 2;    // acc[128], m, l
 constexpr int AT_MAX_SPLITS = 16;    // runs per (b, kv head): the merge loads them all at once
 
+constexpr int DPP_ROW_MIRROR = 0x140;       // lane i <- lane 15 - i  (i ^ 15)
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;  // lane i <- lane 7 - i within 8 lanes  (i ^ 7)
+constexpr int DPP_QUAD_XOR3 = 0x1B;         // quad_perm:[3,2,1,0]
+
+template <int G> struct attn_shape {
+    static_assert(G >= 1 && G <= 8, "query heads per kv head");
+    static constexpr int GP = G <= 2 ? 2 : G <= 4 ? 4 : 8;  // heads, padded to a power of two
+    static constexpr int U = 16 / GP;                       // rows a 16-lane group scores per chunk
+};
+
 template <int G, int NW>
 struct attn_shared {
-    static constexpr int NLG = NW * 4;  // 16-lane groups in the workgroup
-    float m[NLG][G], l[NLG][G], w[(NLG > AT_MAX_SPLITS ? NLG : AT_MAX_SPLITS)][G], M[G], L[G];
-    alignas(16) float acc[NLG][G][AT_D];
+    static constexpr int GP = attn_shape<G>::GP, U = attn_shape<G>::U;
+    static constexpr int NLG = NW * 4;    // 16-lane groups in the workgroup
+    static constexpr int CH = NLG * U;    // rows per chunk
+    static constexpr int RW = CH / NW;    // rows of a chunk one wave accumulates
+    alignas(16) float p[CH][GP];
+    alignas(16) float wmax[NW][GP];
+    alignas(16) float acc[NW][G][AT_D];
+    alignas(16) float l[NW][GP];
+    float M[GP], L[G];
+    float w[AT_MAX_SPLITS][G];
     int last;
 };
 
-// Attends over the rows listed in s_row[0 .. n_rows) (LDS; negative = unused; readable
-// and negative up to the next multiple of NW*4*U), as run `split` of `S` runs of the
-// (b, kv head).  Every lane of the workgroup must call it; the caller has already
-// synchronised the writes to s_row.
-template <typename T, int G, int NW, int U>
+// ---- element-type specifics ---------------------------------------------------------
+
+// Eight consecutive elements as loaded (16-bit types: four packed words).
+template <typename T> struct slice8 { uint4 w; };
+template <> struct slice8<float> { float4 a, b; };
+
+template <typename T> __device__ __forceinline__ slice8<T> load_slice8(const T *p) {
+    slice8<T> s;
+    if constexpr (sizeof(T) == 4) {
+        s.a = reinterpret_cast<const float4 *>(p)[0];
+        s.b = reinterpret_cast<const float4 *>(p)[1];
+    } else {
+        s.w = *reinterpret_cast<const uint4 *>(p);
+    }
+    return s;
+}
+
+typedef __bf16 sl_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 sl_f16x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c);
+template <> __device__ __forceinline__ float dot2_acc<bf16_t>(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(sl_bf16x2, a), __builtin_bit_cast(sl_bf16x2, b), c, false);
+}
+template <> __device__ __forceinline__ float dot2_acc<f16_t>(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(sl_f16x2, a), __builtin_bit_cast(sl_f16x2, b), c, false);
+}
+
+template <typename T> __device__ __forceinline__ float dot_slice8(const slice8<T> &a, const slice8<T> &b) {
+    if constexpr (sizeof(T) == 4) {
+        float d = a.a.x * b.a.x;
+        d = fmaf(a.a.y, b.a.y, d); d = fmaf(a.a.z, b.a.z, d); d = fmaf(a.a.w, b.a.w, d);
+        d = fmaf(a.b.x, b.b.x, d); d = fmaf(a.b.y, b.b.y, d); d = fmaf(a.b.z, b.b.z, d);
+        return fmaf(a.b.w, b.b.w, d);
+    } else {
+        float d = dot2_acc<T>(a.w.x, b.w.x, 0.f);
+        d = dot2_acc<T>(a.w.y, b.w.y, d);
+        d = dot2_acc<T>(a.w.z, b.w.z, d);
+        return dot2_acc<T>(a.w.w, b.w.w, d);
+    }
+}
+
+// Two consecutive elements as loaded, and as fp32.
+template <typename T> struct pair_raw { uint32_t w; };
+template <> struct pair_raw<float> { float2 v; };
+
+template <typename T> __device__ __forceinline__ pair_raw<T> load_pair(const T *p) {
+    pair_raw<T> r;
+    if constexpr (sizeof(T) == 4) r.v = *reinterpret_cast<const float2 *>(p);
+    else r.w = *reinterpret_cast<const uint32_t *>(p);
+    return r;
+}
+
+template <typename T> __device__ __forceinline__ void unpack_pair(const pair_raw<T> &r, float &lo, float &hi) {
+    if constexpr (sizeof(T) == 4) { lo = r.v.x; hi = r.v.y; }
+    else unpack2<T>(r.w, lo, hi);
+}
+
+// ---- cross-lane pieces -----------------------------------------------------------------
+
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(dpp_i32<CTRL>(0, __float_as_int(v)));
+}
+
+// v[i] holds this lane's partial of value i (16 values).  Returns, in lane `sub` of
+// every aligned group of 16 lanes, the sum of value `sub` over the group.  Each
+// step pairs lanes whose index differs in one more bit (and, harmlessly, in lower
+// ones); a lane keeps the half of its values that matches its own bit and adds
+// the partner's copy of that half, so the value count halves while the lane count
+// summed over doubles.
+__device__ __forceinline__ float row16_transpose_sum(float (&v)[16], int sub) {
+    {
+        const bool hi = (sub & 8) != 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float keep = hi ? v[i + 8] : v[i], send = hi ? v[i] : v[i + 8];
+            v[i] = keep + dpp_f32<DPP_ROW_MIRROR>(send);
+        }
+    }
+    {
+        const bool hi = (sub & 4) != 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float keep = hi ? v[i + 4] : v[i], send = hi ? v[i] : v[i + 4];
+            v[i] = keep + dpp_f32<DPP_ROW_HALF_MIRROR>(send);
+        }
+    }
+    {
+        const bool hi = (sub & 2) != 0;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float keep = hi ? v[i + 2] : v[i], send = hi ? v[i] : v[i + 2];
+            v[i] = keep + dpp_f32<DPP_QUAD_XOR3>(send);
+        }
+    }
+    const bool hi = (sub & 1) != 0;
+    const float keep = hi ? v[1] : v[0], send = hi ? v[0] : v[1];
+    return keep + dpp_f32<DPP_QUAD_XOR1>(send);
+}
+
+// Maximum over the lanes of a wave that hold the same head: U consecutive lanes in
+// each of the four 16-lane groups.
+template <int U> __device__ __forceinline__ float head_max(float v) {
+    if constexpr (U >= 2) v = fmaxf(v, dpp_f32<DPP_QUAD_XOR1>(v));
+    if constexpr (U >= 4) v = fmaxf(v, dpp_f32<DPP_QUAD_XOR2>(v));
+    if constexpr (U >= 8) v = fmaxf(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v));  // the quads are uniform by now
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+// Attends over the rows listed in s_row[0 .. n_rows) (LDS; negative = skipped), as
+// run `split` of `S` runs of the (b, kv head).  Every lane of the workgroup must
+// call it; the caller has already synchronised the writes to s_row.
+template <typename T, int G, int NW>
 __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b, int h, int split, int S,
                                                       const int *s_row, int n_rows, attn_shared<G, NW> &sh) {
-    constexpr int NT = NW * 64;
-    constexpr int NLG = NW * 4;
+    using SH = attn_shared<G, NW>;
+    constexpr int NT = NW * 64, NLG = SH::NLG, GP = SH::GP, U = SH::U, CH = SH::CH, RW = SH::RW;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
-    const int sub = lane & 15;            // which 8-element slice of the row
+    const int sub = lane & 15;            // slice of the row in the score phase; value index after the butterfly
     const int rslot = wave * 4 + (lane >> 4);
+    const int g_l = sub / U, u_l = sub % U;  // the (head, row) whose score this lane ends up with
 
     const T *qb = static_cast<const T *>(a.q) + static_cast<int64_t>(b) * a.q_stride_b +
                   static_cast<int64_t>(h) * G * AT_D + sub * 8;
-    float qf[G][8];
+    slice8<T> qs[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        load8<T>(qb + g * AT_D, qf[g]);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) qf[g][j] *= a.scale;
-    }
+    for (int g = 0; g < G; ++g) qs[g] = load_slice8<T>(qb + g * AT_D);
     const T *kb = static_cast<const T *>(a.keys) + static_cast<int64_t>(b) * a.kv_stride_b +
                   static_cast<int64_t>(h) * a.kv_stride_h + sub * 8;
     const T *vb = static_cast<const T *>(a.vals) + static_cast<int64_t>(b) * a.kv_stride_b +
-                  static_cast<int64_t>(h) * a.kv_stride_h + sub * 8;
+                  static_cast<int64_t>(h) * a.kv_stride_h + lane * 2;
 
-    float m[G], l[G], acc[G][8];
+    float m_run[GP], lsum[G], acc[G][2];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        m[g] = -INFINITY;
-        l[g] = 0.f;
+    for (int g = 0; g < GP; ++g) m_run[g] = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[g][j] = 0.f;
+    for (int g = 0; g < G; ++g) { lsum[g] = 0.f; acc[g][0] = 0.f; acc[g][1] = 0.f; }
+
+    for (int base = 0; base < n_rows; base += CH) {
+        // every load of the chunk first: U key slices for the score phase, RW value
+        // pairs for the accumulation phase (an absent or skipped row re-reads row 0
+        // and gets probability 0): no branch sits between the loads
+        int row[U];
+        slice8<T> ks[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int ri = base + u * NLG + rslot;
+            row[u] = ri < n_rows ? s_row[ri] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            ks[u] = load_slice8<T>(kb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n);
+        pair_raw<T> vs[RW];
+#pragma unroll
+        for (int j = 0; j < RW; ++j) {
+            const int ri = base + wave + NW * j;
+            int r = ri < n_rows ? s_row[ri] : -1;
+            r = __builtin_amdgcn_readfirstlane(r >= 0 ? r : 0);  // the same row for the whole wave
+            vs[j] = load_pair<T>(vb + static_cast<int64_t>(r) * a.kv_stride_n);
+        }
+
+        // scores: partial dot products of this lane's slice, then the butterfly
+        float part[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int g = i / U, u = i % U;
+            part[i] = g < G ? dot_slice8<T>(qs[g < G ? g : 0], ks[u]) : 0.f;
+        }
+        float s = row16_transpose_sum(part, sub) * a.scale;
+        int my_row = row[0];
+#pragma unroll
+        for (int u = 1; u < U; ++u) my_row = u_l == u ? row[u] : my_row;
+        const bool valid = my_row >= 0 && g_l < G;
+        s = valid ? s : -INFINITY;
+
+        // chunk maximum per head: in the wave, then over the waves through LDS
+        const float wm = head_max<U>(s);
+        if (lane < 16 && u_l == 0) sh.wmax[wave][g_l] = wm;
+        __syncthreads();
+        float m_new[GP];
+#pragma unroll
+        for (int g = 0; g < GP; ++g) m_new[g] = m_run[g];
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+#pragma unroll
+            for (int g = 0; g < GP; ++g) m_new[g] = fmaxf(m_new[g], sh.wmax[w][g]);
+        float my_m = m_new[0];
+#pragma unroll
+        for (int g = 1; g < GP; ++g) my_m = g_l == g ? m_new[g] : my_m;
+        const float p = valid ? __expf(s - my_m) : 0.f;  // a valid score makes my_m finite
+        sh.p[u_l * NLG + rslot][g_l] = p;
+        __syncthreads();
+
+        // values: rescale what earlier chunks left (exp(-inf) = 0 on the first), then
+        // accumulate this wave's rows of the chunk
+        if (base > 0) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float al = m_run[g] == -INFINITY ? 0.f : __expf(m_run[g] - m_new[g]);
+                lsum[g] *= al; acc[g][0] *= al; acc[g][1] *= al;
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < GP; ++g) m_run[g] = m_new[g];
+#pragma unroll
+        for (int j = 0; j < RW; ++j) {
+            const int rc = wave + NW * j;
+            if (base + rc >= n_rows) break;  // uniform in the wave
+            float v0, v1;
+            unpack_pair<T>(vs[j], v0, v1);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float pg = sh.p[rc][g];
+                lsum[g] += pg;
+                acc[g][0] = fmaf(pg, v0, acc[g][0]);
+                acc[g][1] = fmaf(pg, v1, acc[g][1]);
+            }
+        }
+        if (base + CH < n_rows) __syncthreads();  // the next chunk rewrites wmax and p
     }
 
-    for (int base = 0; base < n_rows; base += NLG * U) {
-        int row[U];
-        float kf[U][8], vf[U][8];
+    // the waves' tiles meet in LDS
 #pragma unroll
-        for (int u = 0; u < U; ++u) row[u] = s_row[base + u * NLG + rslot];
-        // unconditional loads (an unused slot re-reads row 0 and is masked below):
-        // no branch sits between the 2 * U loads
+    for (int g = 0; g < G; ++g) *reinterpret_cast<float2 *>(&sh.acc[wave][g][lane * 2]) = make_float2(acc[g][0], acc[g][1]);
+    if (lane == 0) {
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-            load8<T>(kb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n, kf[u]);
+        for (int g = 0; g < G; ++g) sh.l[wave][g] = lsum[g];
+        if (wave == 0) {
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-            load8<T>(vb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n, vf[u]);
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            float s[U];
-            float mn = m[g];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                float d = 0.f;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) d = fmaf(qf[g][j], kf[u][j], d);
-                d = row16_sum(d);
-                s[u] = row[u] >= 0 ? d : -INFINITY;
-                mn = fmaxf(mn, s[u]);
-            }
-            if (mn == -INFINITY) continue;  // nothing seen yet (uniform within the 16-lane group)
-            const float sc = __expf(m[g] - mn);  // exp(-inf) = 0 on the first rows
-            float p[U], ps = 0.f;
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                p[u] = __expf(s[u] - mn);
-                ps += p[u];
-            }
-            l[g] = fmaf(l[g], sc, ps);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                float t = acc[g][j] * sc;
-#pragma unroll
-                for (int u = 0; u < U; ++u) t = fmaf(p[u], vf[u][j], t);
-                acc[g][j] = t;
-            }
-            m[g] = mn;
+            for (int g = 0; g < G; ++g) sh.M[g] = m_run[g];
         }
     }
-
-    // every 16-lane group parks its state in LDS; wave w turns the states of heads
-    // w, w+NW, .. into one weight exp(m - M) per group plus the head's max and sum
-    if (sub == 0) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) { sh.m[rslot][g] = m[g]; sh.l[rslot][g] = l[g]; }
-    }
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        float4 *dst = reinterpret_cast<float4 *>(&sh.acc[rslot][g][sub * 8]);
-        dst[0] = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
-        dst[1] = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
-    }
     __syncthreads();
-    for (int g = wave; g < G; g += NW) {
-        const float mine = lane < NLG ? sh.m[lane][g] : -INFINITY;
-        const float M = wave_max(mine);
-        const float w = mine == -INFINITY ? 0.f : __expf(mine - M);
-        const float L = wave_sum(lane < NLG ? sh.l[lane][g] * w : 0.f);
-        if (lane < NLG) sh.w[lane][g] = w;
-        if (lane == 0) { sh.M[g] = M; sh.L[g] = L; }
+    if (tid < G) {
+        float L = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) L += sh.l[w][tid];
+        sh.L[tid] = L;
     }
-    __syncthreads();
 
     const int bh = b * a.KH + h;
     T *ob = static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.QH + static_cast<int64_t>(h) * G) * AT_D;
-    float *part = a.part + (static_cast<int64_t>(bh) * AT_MAX_SPLITS + split) * G * AT_PART;
+    float *part_out = a.part + (static_cast<int64_t>(bh) * AT_MAX_SPLITS + split) * G * AT_PART;
+    if (S == 1) __syncthreads();  // sh.L is read below
     for (int e = tid; e < G * AT_D; e += NT) {
         const int g = e / AT_D, c = e % AT_D;
         float O = 0.f;
 #pragma unroll
-        for (int slot = 0; slot < NLG; ++slot) O = fmaf(sh.acc[slot][g][c], sh.w[slot][g], O);
+        for (int w = 0; w < NW; ++w) O += sh.acc[w][g][c];
         if (S == 1) {
             const float L = sh.L[g];
             ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         } else {
-            st_agent(part + g * AT_PART + c, O);
+            st_agent(part_out + g * AT_PART + c, O);
         }
     }
     if (S == 1) {
@@ -159,8 +325,8 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         return;
     }
     if (tid < G) {
-        st_agent(part + tid * AT_PART + AT_D, sh.M[tid]);
-        st_agent(part + tid * AT_PART + AT_D + 1, sh.L[tid]);
+        st_agent(part_out + tid * AT_PART + AT_D, sh.M[tid]);
+        st_agent(part_out + tid * AT_PART + AT_D + 1, sh.L[tid]);
     }
     publish_wait();
     __syncthreads();
@@ -184,14 +350,16 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             pa[i][sp] = (e < G * AT_D && sp < S) ? v : 0.f;
         }
     }
+    static_assert(AT_MAX_SPLITS == 16, "the runs of a head fit one 16-lane row");
     for (int g = wave; g < G; g += NW) {
+        // lanes 0 .. 15 hold one run each: reductions stay inside the 16-lane row
         const int sp = lane < S ? lane : 0;
         const float *ps = pb + (static_cast<int64_t>(sp) * G + g) * AT_PART;
         const float mraw = ld_agent(ps + AT_D), lraw = ld_agent(ps + AT_D + 1);
         const float mine = lane < S ? mraw : -INFINITY;
-        const float M = wave_max(mine);
+        const float M = row16_max(mine);
         const float w = mine == -INFINITY ? 0.f : __expf(mine - M);
-        const float L = wave_sum(lane < S ? lraw * w : 0.f);
+        const float L = row16_sum(lane < S ? lraw * w : 0.f);
         if (lane < AT_MAX_SPLITS) sh.w[lane][g] = w;
         if (lane == 0) sh.L[g] = L;
     }

@@ -127,6 +127,15 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
+// Maximum over each aligned group of 16 lanes; every lane ends with it.
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, __int_as_float(dpp_i32<DPP_QUAD_XOR1>(0, __float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_i32<DPP_QUAD_XOR2>(0, __float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_i32<DPP_ROW_ROR4>(0, __float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_i32<DPP_ROW_ROR8>(0, __float_as_int(v))));
+    return v;
+}
+
 // Inclusive prefix sum over the 64 lanes of a wave.
 __device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x) {
     int v = static_cast<int>(x);
@@ -207,6 +216,25 @@ __device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t x, uint32_t *wa
     }
     *total = tot;
     return base + inc - x;
+}
+
+// Exclusive prefix sums of two values per thread at once (one barrier).
+// `wave_tot`: 2 * NT/64 words of LDS.
+template <int NT>
+__device__ __forceinline__ void block_exclusive_sum2(uint32_t a, uint32_t b, uint32_t *wave_tot, uint32_t *ea, uint32_t *eb) {
+    constexpr int NW = NT / 64;
+    const uint32_t ia = wave_inclusive_sum(a), ib = wave_inclusive_sum(b);
+    if (lane_id() == 63) { wave_tot[wave_id()] = ia; wave_tot[NW + wave_id()] = ib; }
+    __syncthreads();
+    uint32_t ba = 0, bb = 0;
+    const int w = wave_id();
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+        ba += i < w ? wave_tot[i] : 0u;
+        bb += i < w ? wave_tot[NW + i] : 0u;
+    }
+    *ea = ba + ia - a;
+    *eb = bb + ib - b;
 }
 
 // Block sums of two values at once (one barrier).  `wave_tot`: 2 * NT/64 words of LDS.

@@ -3,7 +3,7 @@
 #pragma once
 #include "common.h"
 
-constexpr int HS_THREADS = 256;
+constexpr int HS_THREADS = 512;
 constexpr int HS_U = 4;  // records per lane: HS_U independent loads in flight
 
 struct hamming_args {

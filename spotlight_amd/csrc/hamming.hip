@@ -2,10 +2,10 @@
 //
 // Codes are token-major [B, n, KH, W] words, so the (token, kv head) pairs of a
 // block of tokens are one contiguous run of W-word records.  A workgroup of
-// 256 lanes takes HS_U * 256 consecutive records; lane l reads records
-// l, l+256, ... with one 4*W-byte load each, so every wave-level load covers a
+// 512 lanes takes HS_U * 512 consecutive records; lane l reads records
+// l, l+512, ... with one 4*W-byte load each, so every wave-level load covers a
 // contiguous 64*4*W bytes and all HS_U loads are in flight before the first
-// popcount.  Because 256 % KH == 0 a lane sees the same kv head in every
+// popcount.  Because 512 % KH == 0 a lane sees the same kv head in every
 // record and keeps that head's G query codes in registers.
 //
 // The fused flavour additionally (1) counts every score into an LDS histogram
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     const int h = tid % KH;
     const int tl = tid / KH;
 
-    // LDS carve-up: [FUSED: 1024 int16 scores][G_T == 0: KH*G*W query words][FUSED: KH*NB bins]
+    // LDS carve-up: [FUSED: HS_THREADS*HS_U int16 scores][G_T == 0: KH*G*W query words][FUSED: KH*NB bins]
     int16_t *sc_lds = reinterpret_cast<int16_t *>(smem);
     uint32_t *q_lds = smem + (FUSED ? HS_THREADS * HS_U / 2 : 0);
     uint32_t *hist = q_lds + (G_T > 0 ? 0 : KH * G * W);
@@ -124,20 +124,21 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
 
     if constexpr (FUSED) {
         __syncthreads();
-        // head-major score rows: T int16 per head, four per lane
-        const int T = tok_per_pass * HS_U;  // = 1024 / KH, a multiple of 4
-        const int e4 = tid * 4;
-        const int hh4 = e4 / T, tt = e4 % T;
-        const int64_t t = t0 + tt;
-        if (t < a.n_cap) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(sc_lds + e4);
-            int16_t *dst = a.out + (static_cast<int64_t>(b) * KH + hh4) * a.n_cap + t;
-            *reinterpret_cast<uint2 *>(dst) = v;
+        // head-major score rows: T int16 per head, written four at a time
+        const int T = tok_per_pass * HS_U;  // a multiple of 4 (HS_THREADS * HS_U / KH, KH | 256)
+        for (int e4 = tid * 4; e4 < HS_THREADS * HS_U; e4 += HS_THREADS * 4) {
+            const int hh4 = e4 / T, tt = e4 % T;
+            const int64_t t = t0 + tt;
+            if (t < a.n_cap) {
+                const uint2 v = *reinterpret_cast<const uint2 *>(sc_lds + e4);
+                int16_t *dst = a.out + (static_cast<int64_t>(b) * KH + hh4) * a.n_cap + t;
+                *reinterpret_cast<uint2 *>(dst) = v;
+            }
         }
         // hist_groups copies of the global histogram spread the same-bin adds of the
         // many workgroups of one (b, kv head) over as many addresses; the copy is
         // picked by token span, which the selector relies on.  Every lane
-        // visits KH*NB/256 bins of the workgroup's table (independent LDS reads) and
+        // visits KH*NB/512 bins of the workgroup's table (independent LDS reads) and
         // adds the non-empty ones; e / NB by multiplication (e * NB < 2^32).
         const int grp = static_cast<int>(t0 / a.hist_span) % a.hist_groups;
         uint32_t *gh = a.hist + (static_cast<int64_t>(b) * KH * a.hist_groups + grp) * NB;

@@ -21,7 +21,6 @@ namespace {
 constexpr int SA_NW = 8;
 constexpr int SA_THREADS = SA_NW * 64;
 constexpr int SA_BLOCK = SA_THREADS * TK_RUN;   // 4096 tokens
-constexpr int SA_U = 4;                         // row groups in flight per iteration (128 rows per workgroup)
 constexpr int SA_MAX_BPT = 2;                   // histogram bins per lane (<= 1024 bins)
 
 template <bool dummy = true> struct sa_static_checks {
@@ -31,8 +30,8 @@ template <bool dummy = true> struct sa_static_checks {
 template <typename T, int G, int NG>
 __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args sa, attn_args aa) {
     __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
-    __shared__ int s_tn[2];
-    __shared__ int32_t s_list[SA_BLOCK + SA_NW * 4 * SA_U];
+    __shared__ int s_tn[4];
+    __shared__ int32_t s_list[SA_BLOCK];
     __shared__ attn_shared<G, SA_NW> sh;
 
     const int tid = threadIdx.x;
@@ -56,22 +55,15 @@ __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args s
     const uint4 v = mask_run(raw, t0, n_b);
 
     int thr, need;
-    find_threshold<SA_THREADS, SA_MAX_BPT>(sa, cnt, mine, k_eff, s_wave, s_tn, thr, need);
-    uint32_t pg, pe, tg, te;
-    before_counts<SA_THREADS, SA_MAX_BPT>(sa, before, thr, pg, pe);
-    block_sum2<SA_THREADS>(pg, pe, s_wave + 32, &tg, &te);
+    uint32_t tg, te;
+    find_threshold<SA_THREADS, SA_MAX_BPT>(sa, cnt, before, mine, k_eff, s_wave, s_tn, thr, need, tg, te);
     int n_kept = 0, first = 0;
     place_block<SA_THREADS, true>(v, t0, thr, need, k_eff, tg, te, s_wave, out, s_list, &n_kept, &first);
 
-    // the list goes out with coalesced stores and is padded to whole iterations of
-    // the attention loop, which then runs over it
-    constexpr int ITER = SA_NW * 4 * SA_U;
-    const int padded = (n_kept + ITER - 1) / ITER * ITER;
+    // the list goes out with coalesced stores; the attention then runs over it
     __syncthreads();
     for (int i = tid; i < n_kept; i += SA_THREADS) out[first + i] = s_list[i];
-    for (int i = n_kept + tid; i < padded; i += SA_THREADS) s_list[i] = -1;
-    __syncthreads();
-    attend_rows_and_merge<T, G, SA_NW, SA_U>(aa, b, h, blk, S, s_list, n_kept, sh);
+    attend_rows_and_merge<T, G, SA_NW>(aa, b, h, blk, S, s_list, n_kept, sh);
 }
 
 template <typename T, int G>

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(SH_THREADS) void score_hist_kernel(select_args a, i
 template <bool CONTIG, int MAX_BPT, int NG>
 __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a) {
     __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
-    __shared__ int s_tn[2];
+    __shared__ int s_tn[4];
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.KH, h = bh % a.KH;
@@ -105,10 +105,8 @@ __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a)
     const uint4 v = mask_run(raw, t0, n_b);
 
     int thr, need;
-    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
-    uint32_t pg, pe, tg, te;
-    before_counts<TK_THREADS, MAX_BPT>(a, before, thr, pg, pe);
-    block_sum2<TK_THREADS>(pg, pe, s_wave + 32, &tg, &te);
+    uint32_t tg, te;
+    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, before, mine, k_eff, s_wave, s_tn, thr, need, tg, te);
     const uint32_t uneed = static_cast<uint32_t>(need);
     if (tg + (te < uneed ? te : uneed) >= static_cast<uint32_t>(k_eff)) return;  // everything already placed
     place_block<TK_THREADS>(v, t0, thr, need, k_eff, tg, te, s_wave, out);
@@ -119,7 +117,7 @@ __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a)
 template <bool CONTIG, int MAX_BPT, int NG>
 __global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a) {
     __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
-    __shared__ int s_tn[2];
+    __shared__ int s_tn[4];
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.KH, h = bh % a.KH;
@@ -133,7 +131,8 @@ __global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a)
     const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
     const uint4 v = mask_run(raw, t0, n_b);
     int thr, need;
-    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, mine, k_eff, s_wave, s_tn, thr, need);
+    uint32_t tg_unused, te_unused;
+    find_threshold<TK_THREADS, MAX_BPT>(a, cnt, before, mine, k_eff, s_wave, s_tn, thr, need, tg_unused, te_unused);
     if (blk == 0 && tid == 0) {
         a.thr_need[bh * 2] = thr;
         a.thr_need[bh * 2 + 1] = need;

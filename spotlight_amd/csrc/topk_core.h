@@ -101,44 +101,39 @@ __device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, int 
     return mine;
 }
 
-// Tokens above / at the threshold in front of the block, from the `before` sums of
-// load_bins: per-lane contributions, to be added up over the workgroup.
-template <int NT, int MAX_BPT>
-__device__ __forceinline__ void before_counts(const select_args &a, const uint32_t (&before)[MAX_BPT], int thr,
-                                              uint32_t &above, uint32_t &equal) {
-    const int NB = a.n_bins, tid = threadIdx.x;
-    const int BPT = (NB + NT - 1) / NT;
-    above = 0;
-    equal = 0;
-#pragma unroll
-    for (int j = 0; j < MAX_BPT; ++j) {
-        const int bin = NB - 1 - (tid * BPT + j);
-        above += bin > thr ? before[j] : 0u;
-        equal += bin == thr ? before[j] : 0u;
-    }
-}
-
-// Block-wide search of the threshold bin; every lane returns (thr, need).
+// Block-wide search of the threshold bin; every lane returns (thr, need) and, from
+// the `before` sums of load_bins, the tokens above / at the threshold in front of
+// the block (tg, te).  Both running sums come out of one scan.  s_wave: 32 words,
+// s_tn: 4 words of LDS.
 template <int NT, int MAX_BPT>
 __device__ __forceinline__ void find_threshold(const select_args &a, const uint32_t (&cnt)[MAX_BPT],
-                                               uint32_t mine, int k_eff, uint32_t *s_wave, int *s_tn,
-                                               int &thr, int &need) {
+                                               const uint32_t (&before)[MAX_BPT], uint32_t mine, int k_eff,
+                                               uint32_t *s_wave, int *s_tn, int &thr, int &need,
+                                               uint32_t &tg, uint32_t &te) {
     const int NB = a.n_bins, tid = threadIdx.x;
     const int BPT = (NB + NT - 1) / NT;
-    if (tid == 0) { s_tn[0] = NB; s_tn[1] = 0; }  // selects nothing unless a lane finds the bin
-    uint32_t total;
-    uint32_t cum = block_exclusive_sum<NT>(mine, s_wave, &total);
+    if (tid == 0) { s_tn[0] = NB; s_tn[1] = 0; s_tn[2] = 0; s_tn[3] = 0; }  // selects nothing unless a lane finds the bin
+    uint32_t mine_before = 0;
+#pragma unroll
+    for (int j = 0; j < MAX_BPT; ++j) mine_before += before[j];
+    uint32_t cum, cum_before;
+    block_exclusive_sum2<NT>(mine, mine_before, s_wave, &cum, &cum_before);
 #pragma unroll
     for (int j = 0; j < MAX_BPT; ++j) {
         if (k_eff > 0 && cum < static_cast<uint32_t>(k_eff) && cum + cnt[j] >= static_cast<uint32_t>(k_eff)) {
             s_tn[0] = NB - 1 - (tid * BPT + j);
             s_tn[1] = k_eff - static_cast<int>(cum);
+            s_tn[2] = static_cast<int>(cum_before);
+            s_tn[3] = static_cast<int>(before[j]);
         }
         cum += cnt[j];
+        cum_before += before[j];
     }
     __syncthreads();
     thr = s_tn[0];
     need = s_tn[1];
+    tg = static_cast<uint32_t>(s_tn[2]);
+    te = static_cast<uint32_t>(s_tn[3]);
 }
 
 __device__ __forceinline__ uint32_t count_run(const uint4 &r, int thr) {
