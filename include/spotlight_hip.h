@@ -47,7 +47,8 @@ int sl_version(void);
  * "attn_target_wgs": workgroups the attention launch aims for (default 256);
  * it decides into how many runs the selected rows of a (b, kv head) are cut;
  * "fuse_select_attend": 1 (default) lets the decode step run selection and
- * attention as one launch when the shapes allow, 0 keeps them apart;
+ * attention as one launch when the shapes allow and every 4096-token block keeps
+ * at most 128 rows on average, 2 whenever the shapes allow, 0 never;
  * "hist_copies": copies of the score histogram (4 or 16; 0 = by cache
  * length), to be set before any workspace is sized. */
 int sl_tune(const char *key, int value);

@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, ui
     if (i < n_tail) tail[i] = 0;
 }
 
-int g_fuse_select_attend = 1;  // sl_tune("fuse_select_attend", 0 | 1)
+int g_fuse_select_attend = 1;  // sl_tune("fuse_select_attend", 0 | 1 | 2): never, by shape, whenever possible
 
 struct ws_layout {
     size_t q_code, select, score, attn, total;
@@ -82,7 +82,7 @@ extern "C" int sl_version(void) { return 100; }
 
 extern "C" int sl_tune(const char *key, int value) {
     SL_REQUIRE(key, SL_ERR_NULL);
-    if (!strcmp(key, "fuse_select_attend")) { g_fuse_select_attend = value != 0; return SL_OK; }
+    if (!strcmp(key, "fuse_select_attend") && value >= 0 && value <= 2) { g_fuse_select_attend = value; return SL_OK; }
     const int rc = sl_attn_tune(key, value);
     return rc == SL_OK ? rc : sl_select_tune(key, value);
 }
@@ -176,7 +176,12 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     aa.kv_stride_b = p.n_cap * p.KH * p.d; aa.kv_stride_h = p.d;
     aa.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
     const bool both = (stages & SL_STAGE_SELECT) && (stages & SL_STAGE_ATTN);
-    if (both && p.lru_C == 0 && g_fuse_select_attend && sl_select_attend_supported(ta, aa))
+    // The fused tail attends per 4096-token block.  With few blocks and many kept
+    // rows each workgroup would gather hundreds of rows by itself; the separate
+    // attention launch cuts the rows into more runs than there are blocks then.
+    const int64_t tail_blocks = (p.n_max + 4095) / 4096;
+    const bool fuse_tail = g_fuse_select_attend == 2 || (g_fuse_select_attend == 1 && p.k <= 128 * tail_blocks);
+    if (both && p.lru_C == 0 && fuse_tail && sl_select_attend_supported(ta, aa))
         return sl_select_attend_launch(ta, aa, ws + L.attn, L.total - L.attn, s);
     if (stages & SL_STAGE_SELECT) {
         rc = sl_select_launch(ta, s);
