@@ -217,7 +217,9 @@ def main():
         ab["select+attn"] = ab["attn"]
         # the step runs selection and attention as one launch when it can (no LRU, <= 64k rows):
         # then "select+attn" is that launch and "select" / "attn" are the two-launch alternative
-        fused_tail = not c["lru"] and raw["select+attn"] < 0.9 * (raw["select"] + raw["attn"])
+        # (same rule as the library: the shape allows it and a 4096-token block keeps <= 128 rows on average)
+        fused_tail = (not c["lru"] and n_cap <= 65536 and QH // KH in (1, 2, 4)
+                      and k <= 128 * ((n_max + 4095) // 4096))
         names = ("hash", "score", "select+attn") if fused_tail else ("hash", "score", "select", "lru", "attn")
         for name in ("hash", "score", "select", "lru", "attn", "select+attn"):
             if name in raw:
@@ -228,11 +230,7 @@ def main():
         dominant = max((n for n in kernels if kernels[n]["in_step"] and kernels[n]["algorithmic_bytes"] > 0),
                        key=lambda n: kernels[n]["us"])
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
-    if dominant and os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get(args.config, {}).get(dominant)
+    traffic = profiled_traffic(args.config, dominant) if dominant else None
     roofline = None
     if dominant:
         ach = kernels[dominant]["gbps"]
@@ -262,6 +260,30 @@ def main():
         "kernels": kernels, "roofline": roofline, "cpu_baseline": cpu_baseline,
     }
     print(json.dumps(out), flush=True)
+
+
+STAGE_KERNEL = {"hash": "hash_kernel", "score": "hamming_kernel", "select": "select_fused_kernel",
+                "lru": "lru_kernel", "attn": "sparse_attn_kernel", "select+attn": "select_attend_kernel"}
+
+
+def profiled_traffic(config, stage):
+    """HBM bytes per launch of the stage's kernel as counted by rocprofv3 (FETCH_SIZE and
+    WRITE_SIZE, calibrated on a device copy): read from the committed summary of that
+    profile, profiles/decode_step_<config>_*.txt; None when there is no such summary."""
+    import glob
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", f"decode_step_{config}_*.txt"))):
+        in_table = False
+        with open(path) as f:
+            for line in f:
+                if line.startswith("HBM traffic per launch"):
+                    in_table = True
+                elif in_table and line.startswith(STAGE_KERNEL.get(stage, "?")):
+                    cols = line.split()
+                    try:
+                        return int(round((float(cols[-2]) + float(cols[-1])) * 1e6))
+                    except ValueError:
+                        return None
+    return None
 
 
 def cpu_leg(st, c, budget_s):
