@@ -41,6 +41,7 @@ import torch
 
 from .. import kernel as K
 from ..decode import HashWeights, LayerDecodeState
+from ..modifier import Modifier
 
 
 class MLPLayer(torch.nn.Module):
@@ -234,3 +235,202 @@ def patch_attention(attn_module: torch.nn.Module, layer_idx: int, draft_kwargs: 
     if gqa_key_hash and cfg.num_key_value_heads != cfg.num_attention_heads:
         attn_module.hash_fn_k = MLPHashingFunction(info, cfg.num_key_value_heads, n_layers, mlp_dims, residue)
     attn_module.forward = types.MethodType(self_attn_forward, attn_module)
+
+
+# ---- the objects above the attention forward -----------------------------------------
+# Same names, call signatures and return conventions as the reference's
+# (spotlight_generation.py:24-106, 258-495); the per-layer cache handle is the
+# opaque object ``self_attn_forward`` returns.
+
+class CausalOutput:
+    """What ``model_forward`` returns: the three fields of transformers'
+    ``CausalLMOutputWithPast`` the reference's callers read (:57-60, :478, :487)."""
+
+    def __init__(self, loss, logits, past_key_values):
+        self.loss, self.logits, self.past_key_values = loss, logits, past_key_values
+
+
+def model_forward(self, input_ids, labels=None, kv_cache=None, **kwargs):
+    """spotlight_generation.py:24-60: logits of the LAST position only, as fp32."""
+    hidden_states, kv_cache = self.model(input_ids=input_ids, kv_cache=kv_cache)
+    logits = self.lm_head(hidden_states[..., -1:, :]).float()
+    loss = None
+    if labels is not None:
+        shift_logits = logits[..., :-1, :].reshape(-1, self.config.vocab_size)
+        shift_labels = labels[..., 1:].reshape(-1).to(shift_logits.device)
+        loss = torch.nn.functional.cross_entropy(shift_logits, shift_labels)
+    return CausalOutput(loss, logits, kv_cache)
+
+
+def model_model_forward(self, input_ids=None, kv_cache=None):
+    """spotlight_generation.py:63-79."""
+    hidden_states = self.embed_tokens(input_ids)
+    if kv_cache is None:
+        kv_cache = [None] * len(self.layers)
+    for layer_idx, decoder_layer in enumerate(self.layers):
+        hidden_states, kv_cache[layer_idx] = decoder_layer(hidden_states, kv_cache[layer_idx])
+    return self.norm(hidden_states), kv_cache
+
+
+def layer_forward(self, hidden_states, kv_cache=None):
+    """spotlight_generation.py:82-106."""
+    device = self.self_attn.q_proj.weight.data.device
+    if hidden_states.device != device:
+        hidden_states = hidden_states.to(device)
+    residual = hidden_states
+    hidden_states, kv_cache = self.self_attn(self.input_layernorm(hidden_states), kv_cache)
+    hidden_states = residual + hidden_states
+    residual = hidden_states
+    hidden_states = self.mlp(self.post_attention_layernorm(hidden_states))
+    return residual + hidden_states, kv_cache
+
+
+class Decoder(torch.nn.Module):
+    """spotlight_generation.py:258-383 without the LoRA branch (``enable_lora`` is
+    False in every generation config of the reference, and ``peft`` is not a
+    dependency here)."""
+
+    hash_kind = "mlp"
+
+    def __init__(self, decoder, draft_kwargs):
+        super().__init__()
+        self.decoder = decoder
+        self.enable_lora = False
+        self.fix_layers = list(draft_kwargs.get("fix_layers", []))
+        self.draft_kwargs = draft_kwargs
+        self.model.forward = types.MethodType(model_forward, self.model)
+        self.model.model.forward = types.MethodType(model_model_forward, self.model.model)
+        for layer_idx, layer in enumerate(self.layers):
+            layer.forward = types.MethodType(layer_forward, layer)
+            self._patch(layer.self_attn, layer_idx)
+
+    def _patch(self, attn, layer_idx):
+        patch_attention(attn, layer_idx, self.draft_kwargs, gqa_key_hash=bool(self.draft_kwargs.get("gqa_key_hash", False)))
+
+    @property
+    def layers(self):
+        return self.decoder.model.layers
+
+    @property
+    def model(self):
+        return self.decoder
+
+    def reset(self):
+        """Nothing to drop: the caches live in the handles ``forward`` returns, not on
+        the modules (the reference deletes ``k_cache`` / ``v_cache`` attributes, :282-286)."""
+
+    def is_benchmark_mode(self):
+        return self.draft_kwargs["bench_mark"]
+
+    def enable_benchmark_mode(self):
+        self.draft_kwargs["bench_mark"] = True
+
+    def disable_benchmark_mode(self):
+        self.draft_kwargs["bench_mark"] = False
+
+    def _hash_modules(self, layer):
+        mods = [layer.self_attn.hash_fn]
+        if getattr(layer.self_attn, "hash_fn_k", None) is not None:
+            mods.append(layer.self_attn.hash_fn_k)
+        return mods
+
+    def layer_ft_params(self, layer=None):
+        """One layer's parameters (dense layers: none, :356-360) or, without an
+        argument, the per-layer lists of every layer."""
+        if layer is not None:
+            lay = self.layers[layer]
+            return [] if lay.self_attn.is_fix_layer else [p for m in self._hash_modules(lay) for p in m.parameters()]
+        return [[p for m in self._hash_modules(lay) for p in m.parameters()] for lay in self.layers]
+
+    def ft_params(self, layer=None):
+        """Every layer's hash parameters, dense layers included (:363-369)."""
+        return [p for ps in self.layer_ft_params() for p in ps]
+
+    def forward(self, input_ids, labels=None, kv_cache=None):
+        return self.decoder(input_ids=input_ids, labels=labels, kv_cache=kv_cache)
+
+
+class Model(torch.nn.Module):
+    """spotlight_generation.py:386-437."""
+
+    def __init__(self, decoder: Decoder):
+        super().__init__()
+        self.decoder = decoder
+
+    def ft_params(self):
+        return self.decoder.ft_params()
+
+    def reset(self):
+        self.decoder.reset()
+
+    def forward(self, input_ids, kv_cache=None, labels=None, local_rank=None, **kwargs):
+        if isinstance(input_ids, list):
+            input_ids = torch.tensor(input_ids, dtype=torch.int64)[None, :]
+            if labels is not None:
+                labels = torch.tensor(labels, dtype=torch.int64)[None, :]
+        if input_ids.ndim == 3:
+            input_ids = input_ids.flatten(0, 1)
+        if labels is not None and labels.ndim == 3:
+            labels = labels.flatten(0, 1)
+        device = torch.device(local_rank) if local_rank is not None else next(iter(self.decoder.parameters())).device
+        return self.decoder(input_ids.to(device), labels=labels, kv_cache=kv_cache)
+
+
+class Spotlight(Modifier):
+    """spotlight_generation.py:440-495: ``Spotlight(model, save_ckp, load_ckp, config)``."""
+
+    decoder_cls = Decoder
+
+    def __init__(self, model, save_ckp, load_ckp, config):
+        torch.nn.Module.__init__(self)   # attributes below are set before Modifier.__init__ loads the checkpoint
+        self.get_conf(config)
+        assert isinstance(self.conf, dict)
+        decoder = Model(self.decoder_cls(model, draft_kwargs=self.conf["draft_kwargs"]))
+        super().__init__(decoder, save_ckp, load_ckp)
+
+    def ft_params(self):
+        return self.model.ft_params()
+
+    def layer_ft_params(self):
+        return self.model.decoder.layer_ft_params()
+
+    def fix_layers(self):
+        return self.model.decoder.fix_layers
+
+    def reset(self):
+        self.model.reset()
+
+    def is_benchmark_mode(self):
+        return self.model.decoder.is_benchmark_mode()
+
+    def enable_benchmark_mode(self):
+        return self.model.decoder.enable_benchmark_mode()
+
+    def disable_benchmark_mode(self):
+        return self.model.decoder.disable_benchmark_mode()
+
+    @torch.no_grad()
+    def generate(self, input_ids, max_new_tokens=128, eos_token_id=(2,)):
+        """Greedy decoding (:470-495).  Batch 1 behaves exactly like the reference
+        (stops at an eos token, which is not appended); a larger batch runs every
+        row for ``max_new_tokens`` steps."""
+        if input_ids.ndim == 3:
+            input_ids = input_ids.flatten(0, 1)
+        device = next(iter(self.model.parameters())).device
+        input_ids = input_ids.to(device)
+        output = self.model(input_ids=input_ids)
+        logits, kv_cache = output.logits, output.past_key_values
+        new_tok = logits[:, -1:].argmax(dim=-1)
+        new_ids = []
+        single = input_ids.shape[0] == 1
+        while len(new_ids) < max_new_tokens:
+            if single and new_tok.ravel().item() in eos_token_id:
+                break
+            new_ids.append(new_tok)
+            output = self.model(input_ids=new_tok, kv_cache=kv_cache)
+            logits, kv_cache = output.logits, output.past_key_values
+            new_tok = logits[:, -1:].argmax(dim=-1)
+        self.model.reset()
+        if not new_ids:
+            return input_ids
+        return torch.cat([input_ids] + [t.to(input_ids.dtype) for t in new_ids], dim=-1)
