@@ -213,6 +213,11 @@ def self_attn_forward(self, hidden_states: torch.Tensor, kv_cache=None):
             st.set_k(k)
         out = st.step(ques[:, 0].contiguous(), keys[:, 0].contiguous(), vals[:, 0].contiguous()).unsqueeze(1)
         kv_cache.length = n
+        if dk.get("bench_mark", False):
+            # benchmark mode (spotlight_evaluation.py:303-316): IoU of the selected rows
+            # against the true top-k of q.k, per query head, averaged over the batch
+            from ..iou import selection_iou
+            self.ratios = selection_iou(st.selected(), ques[:, 0], kv_cache.keys[:, :n], k).mean(dim=0).tolist()
 
     attn_output = self.o_proj(out.reshape(B, t, hidden))
     return attn_output, kv_cache
@@ -327,6 +332,18 @@ class Decoder(torch.nn.Module):
 
     def disable_benchmark_mode(self):
         self.draft_kwargs["bench_mark"] = False
+
+    def get_ratios(self, reset=False):
+        """Per layer the IoU list of the last benchmark-mode decode step, None for dense
+        layers (spotlight_generation.py:344-353)."""
+        ratios = []
+        for layer in self.layers:
+            if layer.self_attn.is_fix_layer or not hasattr(layer.self_attn, "ratios"):
+                ratios.append(None)
+            else:
+                ratios.append(layer.self_attn.ratios)
+                del layer.self_attn.ratios
+        return ratios
 
     def _hash_modules(self, layer):
         mods = [layer.self_attn.hash_fn]

@@ -227,3 +227,27 @@ def test_linear_hashing_modifier(mods):
     assert out.past_key_values[1].state.current_k == orc.num_remain(91, 0.9, 8)
     with pytest.raises(NotImplementedError):
         mods("upperbound-generation")
+
+
+@torch.no_grad()
+def test_benchmark_mode_reports_iou_per_layer_and_head(mods):
+    conf = copy.deepcopy(CONF)
+    conf["draft_kwargs"]["bench_mark"] = True
+    base = TinyLM(4, 2, 3, seed=10)
+    m = _wrap(mods, "spotlight-generation", base, conf)
+    assert m.is_benchmark_mode()
+    ids = torch.randint(0, 97, (1, 150), generator=torch.Generator().manual_seed(11))
+    out = m(input_ids=ids.to(DEV))
+    out = m(input_ids=ids[:, :1].to(DEV), kv_cache=out.past_key_values)
+    ratios = m.model.decoder.get_ratios(reset=True)
+    assert ratios[0] is None and len(ratios[1]) == 4 and len(ratios[2]) == 4
+    assert all(0.0 <= r <= 1.0 for row in ratios[1:] for r in row)
+    assert m.model.decoder.get_ratios() == [None, None, None]         # consumed
+    # a budget that covers the whole context selects what the true scores select
+    conf["draft_kwargs"]["min_remain"] = 10 ** 6
+    m2 = _wrap(mods, "spotlight-generation", TinyLM(4, 2, 3, seed=10), conf)
+    out = m2(input_ids=ids.to(DEV))
+    m2(input_ids=ids[:, :1].to(DEV), kv_cache=out.past_key_values)
+    assert all(r == 1.0 for row in m2.model.decoder.get_ratios()[1:] for r in row)
+    m2.disable_benchmark_mode()
+    assert not m2.is_benchmark_mode()
