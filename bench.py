@@ -73,6 +73,8 @@ def main():
                     help="launch heuristic passed to sl_tune (e.g. attn_target_wgs=128)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for HBM byte counters)")
+    ap.add_argument("--host-store", action="store_true",
+                    help="keep the full K/V store in pinned host memory behind the LRU table (configs with LRU slots)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-breakdown", action="store_true")
     args = ap.parse_args()
@@ -121,7 +123,8 @@ def main():
             hq = decode.HashWeights.random_linear(QH, 128, 128, dtype, dev, cpu_gen)
             hk = hq if KH == QH else decode.HashWeights.random_linear(KH, 128, 128, dtype, dev, cpu_gen)
         st = decode.LayerDecodeState(B, QH, KH, d, n_cap, k, hq, hk, dtype=dtype, device=dev,
-                                     lru_slots=c["lru"], inputs=tuple(t[0, li] for t in cur))
+                                     lru_slots=c["lru"], inputs=tuple(t[0, li] for t in cur),
+                                     host_store=args.host_store)
         # prefill in slabs to bound the transient memory of hashing
         st.seq_lens.zero_()
         slab = max(1, (1 << 22) // (B * KH))
@@ -129,7 +132,7 @@ def main():
             s1 = min(n0, s0 + slab)
             kk = torch.randn((B, s1 - s0, KH, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
             vv = torch.randn((B, s1 - s0, KH, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
-            st.keys[:, s0:s1] = kk
+            st.keys[:, s0:s1] = kk      # (a device-to-host copy with --host-store)
             st.vals[:, s0:s1] = vv
             kernel.cache_append(st.codes, st.hash_k.hash_rows(kk), start=s0)
         st.seq_lens.fill_(n0)
@@ -252,7 +255,8 @@ def main():
         "dtype": c["dtype"], "data": "synthetic",
         "config": {"workload": f"{args.config}: {c['desc']}", "batch": B, "q_heads": QH, "kv_heads": KH,
                    "head_dim": d, "context": n0, "k": k, "code_bits": 128, "hash": c["hash"],
-                   "lru_slots": c["lru"], "layers_rotated": L, "graph": "one HIP graph per token"},
+                   "lru_slots": c["lru"], "kv_store": "pinned host memory" if args.host_store else "hbm",
+                   "layers_rotated": L, "graph": "one HIP graph per token"},
         "gpu_event_ms_per_step": round(gpu_ms / steps, 6),
         "hbm_gbps": round(step_gbps, 1), "hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(ab["step"]),

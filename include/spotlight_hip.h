@@ -149,6 +149,17 @@ int sl_cache_append(const void *src, void *dst, int B, int64_t t, int64_t row_by
                     int64_t src_stride_b, int64_t dst_stride_b, int64_t start,
                     const int32_t *seq_lens, void *stream);
 
+/* Host-memory tier.  The reference's CPU cache keeps K and V of the sparse
+ * layers in host memory, moves the scores to the host, selects and gathers
+ * there and copies the selected rows back every step
+ * (spotlight/modifiers/cpu_cache.py:50-57,105-130).  Here the full store may
+ * live in PINNED host memory that the GPU reads and writes in place over the
+ * host link: sl_cache_append, sl_gather_kv, sl_lru_update and the keys / vals
+ * of sl_decode_step take the device-side address of such memory, which this
+ * call returns.  SL_ERR_UNSUPPORTED when host_ptr is not pinned, mapped host
+ * memory (pageable memory must never be handed to a kernel). */
+int sl_host_device_pointer(void *host_ptr, void **device_ptr);
+
 /* LRU resident table; NO counterpart in the reference (its caches are
  * append-only, gpu_cache.py:108-118; cpu_cache.py:105-130 re-fetches every
  * selected row from host memory each step, which this table exists to avoid).

@@ -45,6 +45,7 @@ SIGNATURES = {
     "sl_strerror": (C.c_char_p, [c_int]),
     "sl_version": (c_int, []),
     "sl_tune": (c_int, [C.c_char_p, c_int]),
+    "sl_host_device_pointer": (c_int, [c_void_p, C.POINTER(c_void_p)]),
     "sl_pack_sign_u32": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "sl_pack_sign_u8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "sl_hash_mlp_pack": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_int64] * 4 + [c_void_p, c_void_p]),

@@ -87,6 +87,17 @@ extern "C" int sl_tune(const char *key, int value) {
     return rc == SL_OK ? rc : sl_select_tune(key, value);
 }
 
+extern "C" int sl_host_device_pointer(void *host_ptr, void **device_ptr) {
+    SL_REQUIRE(host_ptr && device_ptr, SL_ERR_NULL);
+    void *dev = nullptr;
+    if (hipHostGetDevicePointer(&dev, host_ptr, 0) != hipSuccess || !dev) {
+        (void)hipGetLastError();  // do not leave the error for the next launch check
+        return SL_ERR_UNSUPPORTED;
+    }
+    *device_ptr = dev;
+    return SL_OK;
+}
+
 extern "C" int sl_workspace_init(void *ws, size_t ws_bytes, void *stream) {
     if (ws_bytes == 0) return SL_OK;
     SL_REQUIRE(ws, SL_ERR_NULL);

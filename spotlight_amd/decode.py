@@ -93,7 +93,7 @@ class HashWeights:
 class LayerDecodeState:
     def __init__(self, batch_size: int, num_heads: int, num_kv_heads: int, head_dim: int, n_cap: int, k: int,
                  hash_q: HashWeights, hash_k: HashWeights, dtype=torch.bfloat16, device="cuda",
-                 head_map: str = "blocked", lru_slots: int = 0, inputs=None):
+                 head_map: str = "blocked", lru_slots: int = 0, inputs=None, host_store: bool = False):
         assert head_dim == 128, "the attention kernel covers head_dim 128"
         assert n_cap % 8 == 0, "n_cap must be a multiple of 8"
         assert hash_q.nbits == hash_k.nbits and hash_q.n_layers == hash_k.n_layers
@@ -107,8 +107,17 @@ class LayerDecodeState:
         dev = self.device
         B, QH, KH, d, W = self.B, self.QH, self.KH, self.d, self.W
         self.codes = torch.zeros((B, n_cap, KH, W), dtype=torch.uint32, device=dev)
-        self.keys = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=dev)
-        self.vals = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=dev)
+        # host_store: the full K / V store lives in pinned host memory, which the step's
+        # kernels append to and fetch missed rows from in place; the GPU then only
+        # holds the codes and the LRU resident table the attention reads
+        self.host_store = host_store
+        if host_store:
+            assert lru_slots, "a host-memory store needs the LRU resident table in front of it"
+            self.keys = torch.zeros((B, n_cap, KH, d), dtype=dtype, pin_memory=True)
+            self.vals = torch.zeros((B, n_cap, KH, d), dtype=dtype, pin_memory=True)
+        else:
+            self.keys = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=dev)
+            self.vals = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=dev)
         self.seq_lens = torch.zeros((B,), dtype=torch.int32, device=dev)
         self.step_counter = torch.zeros((1,), dtype=torch.int32, device=dev)
         if inputs is None:  # the step's inputs are read from these buffers
@@ -155,7 +164,7 @@ class LayerDecodeState:
         ptr = lambda t: t.data_ptr() if t is not None else None
         p.w1_q, p.b1_q, p.w2_q, p.b2_q = ptr(hq.w1), ptr(hq.b1), ptr(hq.w2), ptr(hq.b2)
         p.w1_k, p.b1_k, p.w2_k, p.b2_k = ptr(hk.w1), ptr(hk.b1), ptr(hk.w2), ptr(hk.b2)
-        p.codes, p.keys, p.vals = self.codes.data_ptr(), self.keys.data_ptr(), self.vals.data_ptr()
+        p.codes, p.keys, p.vals = self.codes.data_ptr(), K.device_ptr(self.keys), K.device_ptr(self.vals)
         p.seq_lens, p.out, p.idx = self.seq_lens.data_ptr(), self.out.data_ptr(), self.idx.data_ptr()
         p.step_counter = self.step_counter.data_ptr()
         p.lru_C = self.lru_slots

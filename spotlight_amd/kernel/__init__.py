@@ -46,6 +46,27 @@ def _need_gpu(*ts: torch.Tensor) -> None:
             raise RuntimeError("Input must be on the GPU")
 
 
+def device_ptr(t: torch.Tensor) -> int:
+    """Address a kernel may use for ``t``: its data pointer for a GPU tensor, the
+    device-side address of the mapping for a PINNED host tensor (the host-memory
+    tier; the kernels then read and write host memory in place).  Pageable host
+    memory is refused."""
+    if t.is_cuda:
+        return t.data_ptr()
+    if not t.is_pinned():
+        raise RuntimeError("Input must be on the GPU or in pinned host memory")
+    import ctypes
+    dev = ctypes.c_void_p()
+    _lib.check(_L.sl_host_device_pointer(t.data_ptr(), ctypes.byref(dev)), "sl_host_device_pointer")
+    return dev.value
+
+
+def _need_gpu_or_pinned(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if not t.is_cuda and not t.is_pinned():
+            raise RuntimeError("Input must be on the GPU or in pinned host memory")
+
+
 class Workspace:
     """A zero-initialised scratch buffer the kernels leave zeroed again.
     One per concurrent caller; grown on demand."""
@@ -218,16 +239,17 @@ def gather_kv(keys: torch.Tensor, vals: torch.Tensor, idx: torch.Tensor) -> Tupl
     """keys/vals [B,L,KH,d] (rows contiguous), idx int32 [B,KH,k] ->
     (K_sel, V_sel) [B,k,KH,d]; the two torch.gather calls of
     spotlight/modifiers/gpu_cache.py:51-53."""
-    _need_gpu(keys, vals, idx)
+    _need_gpu(idx)
+    _need_gpu_or_pinned(keys, vals)      # a pinned host store is gathered from in place
     B, L, KH, d = keys.shape
     k = idx.shape[2]
     assert keys.shape == vals.shape and keys.stride() == vals.stride()
     assert keys.stride(3) == 1 and keys.stride(2) == d and keys.stride(1) == KH * d
     assert idx.dtype == torch.int32 and idx.is_contiguous()
-    k_out = torch.empty((B, k, KH, d), dtype=keys.dtype, device=keys.device)
+    k_out = torch.empty((B, k, KH, d), dtype=keys.dtype, device=idx.device)
     v_out = torch.empty_like(k_out)
-    with torch.cuda.device(keys.device):
-        _lib.check(_L.sl_gather_kv(keys.data_ptr(), vals.data_ptr(), idx.data_ptr(), k_out.data_ptr(),
+    with torch.cuda.device(idx.device):
+        _lib.check(_L.sl_gather_kv(device_ptr(keys), device_ptr(vals), idx.data_ptr(), k_out.data_ptr(),
                                    v_out.data_ptr(), _dtype(keys), B, KH, d, k, keys.stride(0), _stream()),
                    "sl_gather_kv")
     return k_out, v_out
@@ -298,16 +320,17 @@ def cache_append(dst: torch.Tensor, src: torch.Tensor, start: int = 0,
                  seq_lens: Optional[torch.Tensor] = None) -> None:
     """dst[b, start + seq_lens[b] : ... + t] = src[b]  for dst [B,L,...] and
     src [B,t,...] with contiguous rows (gpu_cache.py:42,112-113)."""
-    _need_gpu(dst, src)
+    _need_gpu(src)
+    _need_gpu_or_pinned(dst)             # a pinned host store is appended to in place
     B, t = src.shape[0], src.shape[1]
     row_bytes = src[0, 0].numel() * src.element_size()
     assert dst.dtype == src.dtype and dst[0, 0].numel() == src[0, 0].numel()
     assert src[0].is_contiguous() and dst[0].is_contiguous()
     if seq_lens is None and start + t > dst.shape[1]:
         raise RuntimeError("append exceeds the cache capacity")
-    with torch.cuda.device(dst.device):
+    with torch.cuda.device(src.device):
         _lib.check(_L.sl_cache_append(
-            src.data_ptr(), dst.data_ptr(), B, t, row_bytes, src.stride(0) * src.element_size(),
+            src.data_ptr(), device_ptr(dst), B, t, row_bytes, src.stride(0) * src.element_size(),
             dst.stride(0) * dst.element_size(), start,
             seq_lens.data_ptr() if seq_lens is not None else None, _stream()), "sl_cache_append")
 
