@@ -42,6 +42,24 @@ __global__ __launch_bounds__(256) void gather_kernel(const uint4 *__restrict__ k
 }
 
 // ---- LRU ------------------------------------------------------------------------
+constexpr int LRU_CP = 4;  // 16-byte chunks of K and of V a lane keeps in flight while rows are fetched
+
+// The chunks e0 + u*LRU_THREADS + tid (u < LRU_CP) of the missed rows: loads are
+// unconditional (an idle lane re-reads chunk 0 and gets destination -1).
+#define LRU_ISSUE(E0)                                                                              \
+    _Pragma("unroll") for (int u = 0; u < LRU_CP; ++u) {                                           \
+        const int e = (E0) + u * LRU_THREADS + tid;                                                \
+        const int ec = e < n_chunks ? e : 0;                                                       \
+        const int j = ec / CH, c = ec % CH;                                                        \
+        const int64_t src = (static_cast<int64_t>(s_miss_tok[j]) * a.KH + h) * CH + c;             \
+        dsts[u] = e < n_chunks ? s_victim[j] * CH + c : -1;                                        \
+        kbuf[u] = *reinterpret_cast<const u32x4 *>(kf + src);                                                                         \
+        vbuf[u] = *reinterpret_cast<const u32x4 *>(vf + src);                                                                         \
+    }
+#define LRU_RETIRE()                                                                               \
+    _Pragma("unroll") for (int u = 0; u < LRU_CP; ++u)                                             \
+        if (dsts[u] >= 0) { *reinterpret_cast<u32x4 *>(kr + dsts[u]) = kbuf[u]; *reinterpret_cast<u32x4 *>(vr + dsts[u]) = vbuf[u]; }
+
 // One workgroup per (b, kv head).  Wanted tokens are classified against the
 // token -> slot map; the M victims are the M smallest (stamp, slot) among the
 // slots that were not hit, found with a 4 x 8-bit radix select on the stamp and
@@ -134,8 +152,25 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
             elig[j] = j < SPT && s < C && s_flag[s] == 0;
             key[j] = elig[j] ? ss[s] : 0u;
         }
+        // stamps are step numbers: the high bytes are usually all zero, and a radix
+        // pass over a byte that is zero in every key selects nothing -- skip those
+        uint32_t kmax = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) kmax = key[j] > kmax ? key[j] : kmax;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const uint32_t other = static_cast<uint32_t>(__shfl_xor(static_cast<int>(kmax), o, 64));
+            kmax = other > kmax ? other : kmax;
+        }
+        if (tid == 0) s_digit = 0;
+        __syncthreads();
+        if ((tid & 63) == 0) atomicMax(&s_digit, kmax);
+        __syncthreads();
+        const uint32_t all_max = s_digit;
+        const int first_pass = all_max < (1u << 8) ? 3 : all_max < (1u << 16) ? 2 : all_max < (1u << 24) ? 1 : 0;
+        __syncthreads();  // s_digit is rewritten by the passes
         uint32_t prefix = 0, remaining = static_cast<uint32_t>(M);
-        for (int pass = 0; pass < 4; ++pass) {
+        for (int pass = first_pass; pass < 4; ++pass) {
             const int shift = 24 - 8 * pass;
             const uint32_t hi_mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
             if (tid < 256) s_hist[tid] = 0;
@@ -190,9 +225,29 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
         }
         __syncthreads();
 
+        // fetch the missed rows from the full store into their slots: LRU_CP 16-byte
+        // chunks of K and of V per lane are in flight at once, and they are issued
+        // before the bookkeeping below, which does not depend on them
+        const int es = a.dtype == SL_F32 ? 4 : 2;
+        const int CH = a.d * es / 16;
+        const uint4 *kf = static_cast<const uint4 *>(a.keys) + static_cast<int64_t>(b) * a.kv_stride_b * es / 16;
+        const uint4 *vf = static_cast<const uint4 *>(a.vals) + static_cast<int64_t>(b) * a.kv_stride_b * es / 16;
+        uint4 *kr = static_cast<uint4 *>(a.k_res) + bh * C * CH;
+        uint4 *vr = static_cast<uint4 *>(a.v_res) + bh * C * CH;
+        const int n_chunks = M * CH;
+        // (a native vector type: arrays of the HIP uint4 struct were not kept in registers here)
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        u32x4 kbuf[LRU_CP], vbuf[LRU_CP];
+        int dsts[LRU_CP];
+        // (loads return in order: the slot's old token is fetched before the row chunks,
+        // or the bookkeeping would wait for all of them)
+        const bool has_first = tid < M;
+        const int s_first = has_first ? s_victim[tid] : 0;
+        const int old_first = st[s_first];
+        LRU_ISSUE(0)
         for (int j = tid; j < M; j += LRU_THREADS) {
             const int tk = s_miss_tok[j], s = s_victim[j];
-            const int old = st[s];
+            const int old = j == tid ? old_first : st[s];
             if (old >= 0) ts[old] = -1;
             ts[tk] = s;
             st[s] = tk;
@@ -200,21 +255,14 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
             const int item = s_miss_item[j];
             if (item < k) so[item] = s;
         }
-        // fetch the missed rows from the full store into their slots
-        const int es = a.dtype == SL_F32 ? 4 : 2;
-        const int CH = a.d * es / 16;
-        const uint4 *kf = static_cast<const uint4 *>(a.keys) + static_cast<int64_t>(b) * a.kv_stride_b * es / 16;
-        const uint4 *vf = static_cast<const uint4 *>(a.vals) + static_cast<int64_t>(b) * a.kv_stride_b * es / 16;
-        uint4 *kr = static_cast<uint4 *>(a.k_res) + bh * C * CH;
-        uint4 *vr = static_cast<uint4 *>(a.v_res) + bh * C * CH;
-        for (int e = tid; e < M * CH; e += LRU_THREADS) {
-            const int j = e / CH, c = e % CH;
-            const int64_t src = (static_cast<int64_t>(s_miss_tok[j]) * a.KH + h) * CH + c;
-            const int64_t dst = static_cast<int64_t>(s_victim[j]) * CH + c;
-            kr[dst] = kf[src];
-            vr[dst] = vf[src];
+        LRU_RETIRE()
+        for (int e0 = LRU_CP * LRU_THREADS; e0 < n_chunks; e0 += LRU_CP * LRU_THREADS) {
+            LRU_ISSUE(e0)
+            LRU_RETIRE()
         }
     }
+#undef LRU_ISSUE
+#undef LRU_RETIRE
     if (tid == 0 && a.stats) {
         a.stats[bh * 2] += static_cast<uint32_t>(n_wanted - M);
         a.stats[bh * 2 + 1] += static_cast<uint32_t>(M);
