@@ -1,7 +1,7 @@
 // (a) fused hash -> sign -> pack for the decode step's new vectors.
 //
 // Per head the hash is a GEMV against 64-130 KB of weights and the step is
-// latency bound, so one workgroup of 16 waves owns a whole head: every lane
+// latency bound, so one workgroup of 8 waves owns a whole head: every lane
 // issues all its 16-byte weight loads of both projections up front (the whole
 // head is in flight in one memory round trip), the weights stay in registers
 // while the workgroup loops over its batch rows, and nothing has to cross
@@ -9,9 +9,9 @@
 //   projection 1  [d_in=128, d_hid]: lane (cg, r) holds 8 columns of rows
 //                 r, r+RPP, ...; partial sums meet in LDS [RPP][d_hid];
 //   projection 2  [d_hid, 128]: lane (cg2, r2) holds 8 columns of rows
-//                 r2, r2+64, ...; partial sums meet in LDS [64][128];
+//                 r2, r2+R2, ... (R2 = lanes/16); partial sums meet in LDS [R2][128];
 //   both LDS tables hold 8192 partial sums and are folded in two steps by all
-//   1024 lanes (8 rows per lane, then one lane per column adds the 1024/columns
+//   lanes (8 rows per lane, then one lane per column adds the lanes/columns
 //   sub-totals), so no lane walks a long serial chain of LDS reads;
 //   the 128 pre-activations are turned into sign bits with a wave ballot and
 //   stored as packed words straight into their destination (the query-code
@@ -26,7 +26,7 @@
 
 namespace {
 
-constexpr int HK_THREADS = 1024;
+constexpr int HK_THREADS = 512;
 constexpr int HK_DIN = 128;
 constexpr int HK_NBITS = 128;
 constexpr int HK_B_PER_WG = 4;  // batch rows one workgroup loops over
@@ -38,7 +38,7 @@ template <int D_HID> struct l1_shape {
     static constexpr int LPR = D_HID / 8;             // lanes per weight row
     static constexpr int RPP = HK_THREADS / LPR;      // rows per pass
     static constexpr int PASSES = HK_DIN / RPP;       // rows per lane
-    static_assert(PASSES >= 1, "d_hid too small for 1024 lanes");
+    static_assert(PASSES >= 1, "d_hid too small for the workgroup");
     static_assert(RPP * D_HID == HK_THREADS * HK_FOLD, "partial-sum table is 8 entries per lane");
 };
 
@@ -69,7 +69,10 @@ __device__ __forceinline__ float fold_columns(const float *red, float *sub) {
 template <typename T, int NL, int D_HID>
 __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     using S1 = l1_shape<D_HID>;
-    constexpr int P2 = NL == 2 ? D_HID / 64 : 1;     // second projection: 64 rows per pass
+    constexpr int R2 = HK_THREADS / 16;              // second projection: rows per pass (16 lanes per row)
+    constexpr int P2 = NL == 2 ? (D_HID + R2 - 1) / R2 : 1;
+    static_assert(NL == 1 || D_HID % R2 == 0, "hidden width must be whole passes of the second projection");
+    static_assert(R2 * HK_NBITS == HK_THREADS * HK_FOLD, "partial-sum table is 8 entries per lane");
     __shared__ float xs[HK_DIN];
     __shared__ __align__(16) float red[HK_THREADS * HK_FOLD];
     __shared__ float sub[HK_THREADS];
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     if constexpr (NL == 2) {
         const T *w2 = static_cast<const T *>(sd.w2) + static_cast<int64_t>(h) * D_HID * HK_NBITS + cg2 * 8;
 #pragma unroll
-        for (int q = 0; q < P2; ++q) load8<T>(w2 + static_cast<int64_t>(r2 + 64 * q) * HK_NBITS, w2r[q]);
+        for (int q = 0; q < P2; ++q) load8<T>(w2 + static_cast<int64_t>(r2 + R2 * q) * HK_NBITS, w2r[q]);
     }
     // optional operands are loaded without a branch (an absent one re-reads the
     // input row and is ignored): a load under a condition would have to be waited
@@ -191,7 +194,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
                 float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int q = 0; q < P2; ++q) {
-                    const float hv = hidl[r2 + 64 * q];
+                    const float hv = hidl[r2 + R2 * q];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) acc[j] = fmaf(hv, w2r[q][j], acc[j]);
                 }
