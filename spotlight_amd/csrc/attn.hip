@@ -12,8 +12,9 @@
 
 namespace {
 
-constexpr int AT_NW = 4;             // waves per workgroup
-constexpr int AT_THREADS = AT_NW * 64;
+// waves per workgroup: 4 for short runs (one wave per SIMD: the lowest latency), 8 from
+// AT_WIDE_ROWS rows per run on (twice the rows per chunk, half the chunk barriers)
+constexpr int AT_WIDE_ROWS = 128;
 constexpr int AT_ITER_ROWS = 64;     // runs are cut at multiples of this many rows
 constexpr int AT_MAX_ROWS = 1024;    // rows per run (LDS row-number buffer)
 // The arrival tickets sit in a fixed-size head of the workspace so that the
@@ -21,23 +22,27 @@ constexpr int AT_MAX_ROWS = 1024;    // rows per run (LDS row-number buffer)
 // the only part that has to stay zero between calls.
 constexpr size_t AT_COUNTER_BYTES = 64 * 1024;
 
-template <typename T, int G>
-__global__ __launch_bounds__(AT_THREADS) void sparse_attn_kernel(attn_args a) {
+template <typename T, int G, int NW>
+__global__ __launch_bounds__(NW * 64) void sparse_attn_kernel(attn_args a) {
+    constexpr int AT_THREADS = NW * 64;
     __shared__ int s_row[AT_MAX_ROWS];
-    __shared__ attn_shared<G, AT_NW> sh;
+    __shared__ attn_shared<G, NW> sh;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int r_lo = split * a.rows;
     const int r_hi = r_lo + a.rows < a.k ? r_lo + a.rows : a.k;
     const int32_t *idx = a.idx + (static_cast<int64_t>(b) * a.KH + h) * a.k;
     for (int i = threadIdx.x; i < a.rows; i += AT_THREADS) s_row[i] = r_lo + i < r_hi ? idx[r_lo + i] : -1;
     __syncthreads();
-    attend_rows_and_merge<T, G, AT_NW>(a, b, h, split, gridDim.x, s_row, a.rows, sh);
+    attend_rows_and_merge<T, G, NW>(a, b, h, split, gridDim.x, s_row, a.rows, sh);
 }
+
+int g_attn_wide_rows = AT_WIDE_ROWS;  // sl_tune("attn_wide_rows", n)
 
 template <typename T, int G>
 int launch(const attn_args &a, hipStream_t s) {
     const int S = (a.k + a.rows - 1) / a.rows;
-    sparse_attn_kernel<T, G><<<dim3(S, a.KH, a.B), dim3(AT_THREADS), 0, s>>>(a);
+    if (a.rows >= g_attn_wide_rows) sparse_attn_kernel<T, G, 8><<<dim3(S, a.KH, a.B), dim3(512), 0, s>>>(a);
+    else sparse_attn_kernel<T, G, 4><<<dim3(S, a.KH, a.B), dim3(256), 0, s>>>(a);
     return sl_check_launch();
 }
 
@@ -74,6 +79,7 @@ int pick_rows(int B, int KH, int k) {
 
 int sl_attn_tune(const char *key, int value) {
     if (!strcmp(key, "attn_target_wgs") && value > 0) { g_attn_target_wgs = value; return SL_OK; }
+    if (!strcmp(key, "attn_wide_rows") && value > 0) { g_attn_wide_rows = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
 

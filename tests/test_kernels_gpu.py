@@ -230,6 +230,8 @@ ATTN_CASES = [
     (1, 8, 8, 64, 1),
     (3, 16, 8, 200, 33),
     (16, 32, 8, 700, 328),
+    (1, 10, 2, 6000, 2622),     # long runs: the 8-wave flavour, 5 query heads per kv head
+    (1, 4, 4, 3000, 2500),
 ]
 
 
