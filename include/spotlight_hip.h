@@ -51,7 +51,7 @@ int sl_version(void);
  * at most 128 rows on average, 2 whenever the shapes allow, 0 never;
  * "attn_wide_rows": rows per run from which the attention launch uses 8 waves per
  * workgroup instead of 4 (default 128);
- * "hist_copies": copies of the score histogram (4, 16 or 32; 0 = by cache
+ * "hist_copies": copies of the score histogram (4, 8, 16 or 32; 0 = by cache
  * length), to be set before any workspace is sized. */
 int sl_tune(const char *key, int value);
 

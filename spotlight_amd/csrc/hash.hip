@@ -4,7 +4,7 @@
 // latency bound, so one workgroup of 8 waves owns a whole head: every lane
 // issues all its 16-byte weight loads of both projections up front (the whole
 // head is in flight in one memory round trip), the weights stay in registers
-// while the workgroup loops over its batch rows, and nothing has to cross
+// for all batch rows of the workgroup, and nothing has to cross
 // workgroups -- no workspace, no tickets.
 //   projection 1  [d_in=128, d_hid]: lane (cg, r) holds 8 columns of rows
 //                 r, r+RPP, ...; partial sums meet in LDS [RPP][d_hid];
@@ -29,8 +29,12 @@ namespace {
 constexpr int HK_THREADS = 512;
 constexpr int HK_DIN = 128;
 constexpr int HK_NBITS = 128;
-constexpr int HK_B_PER_WG = 4;  // batch rows one workgroup loops over
+constexpr int HK_B_PER_WG = 4;  // batch rows one workgroup takes when the batch is larger than one
 constexpr int HK_FOLD = 8;      // rows of a partial-sum table one lane folds in the first step
+
+__device__ __forceinline__ bool sl_aligned_dev(const void *p, uintptr_t a) {
+    return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
 
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
@@ -42,49 +46,60 @@ template <int D_HID> struct l1_shape {
     static_assert(RPP * D_HID == HK_THREADS * HK_FOLD, "partial-sum table is 8 entries per lane");
 };
 
-// Column sums of the partial-sum table red[ROWS][COLS] (ROWS * COLS = 8192) with
-// all lanes: lane (part, col) adds 8 rows into sub[part][col], then the lanes
-// tid < COLS add the ROWS / 8 sub-totals of their column.  Returns the column sum
-// in lanes tid < COLS (0 elsewhere).  Two barriers; `red` may be rewritten after it.
-template <int COLS>
-__device__ __forceinline__ float fold_columns(const float *red, float *sub) {
+// Column sums of R partial-sum tables red[R][ROWS][COLS] (ROWS * COLS = 8 entries per
+// lane) with all lanes: lane (part, col) adds 8 rows of every table into
+// sub[R][part][col], then the lanes tid < COLS add the ROWS / 8 sub-totals of their
+// column.  total[rr] is the column sum of table rr in lanes tid < COLS (0 elsewhere).
+// One barrier inside; `red` may be rewritten after it.
+template <int COLS, int R>
+__device__ __forceinline__ void fold_columns(const float *red, float *sub, float (&total)[R]) {
     constexpr int PARTS = HK_THREADS / COLS;
+    constexpr int TABLE = HK_THREADS * HK_FOLD;
     const int tid = threadIdx.x;
     const int col = tid % COLS, part = tid / COLS;
-    float s = 0.f;
 #pragma unroll
-    for (int i = 0; i < HK_FOLD; ++i) s += red[(part * HK_FOLD + i) * COLS + col];
-    sub[part * COLS + col] = s;
-    __syncthreads();
-    float total = 0.f;
-    if (tid < COLS) {
+    for (int rr = 0; rr < R; ++rr) {
+        float s = 0.f;
 #pragma unroll
-        for (int i = 0; i < PARTS; ++i) total += sub[i * COLS + tid];
+        for (int i = 0; i < HK_FOLD; ++i) s += red[rr * TABLE + (part * HK_FOLD + i) * COLS + col];
+        sub[rr * HK_THREADS + part * COLS + col] = s;
     }
-    return total;
+    __syncthreads();
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+        total[rr] = 0.f;
+        if (tid < COLS) {
+#pragma unroll
+            for (int i = 0; i < PARTS; ++i) total[rr] += sub[rr * HK_THREADS + i * COLS + tid];
+        }
+    }
 }
 
 // One workgroup of HK_THREADS lanes hashes head blockIdx.x (numbered over both
-// sides) for the batch rows [blockIdx.y * HK_B_PER_WG, ..).
-template <typename T, int NL, int D_HID>
+// sides) for the batch rows [blockIdx.y * R, ..): R = 1 or HK_B_PER_WG rows go
+// through the projections TOGETHER, sharing every barrier and the weights in
+// registers (rows beyond the batch repeat the first row and store nothing).
+template <typename T, int NL, int D_HID, int R>
 __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     using S1 = l1_shape<D_HID>;
     constexpr int R2 = HK_THREADS / 16;              // second projection: rows per pass (16 lanes per row)
     constexpr int P2 = NL == 2 ? (D_HID + R2 - 1) / R2 : 1;
     static_assert(NL == 1 || D_HID % R2 == 0, "hidden width must be whole passes of the second projection");
     static_assert(R2 * HK_NBITS == HK_THREADS * HK_FOLD, "partial-sum table is 8 entries per lane");
-    __shared__ float xs[HK_DIN];
-    __shared__ __align__(16) float red[HK_THREADS * HK_FOLD];
-    __shared__ float sub[HK_THREADS];
-    __shared__ float hidl[D_HID];
+    constexpr int TABLE = HK_THREADS * HK_FOLD;
+    __shared__ float xs[R][HK_DIN];
+    __shared__ __align__(16) float red[R * TABLE];
+    __shared__ float sub[R * HK_THREADS];
+    __shared__ float hidl[R][D_HID];
 
     const int tid = threadIdx.x;
     const int hh = blockIdx.x;
     const int side_i = (a.n_sides > 1 && hh >= a.side[0].H) ? 1 : 0;
     const hash_side &sd = a.side[side_i];
     const int h = hh - (side_i ? a.side[0].H : 0);
-    const int b_lo = blockIdx.y * HK_B_PER_WG;
-    const int b_hi = b_lo + HK_B_PER_WG < a.B ? b_lo + HK_B_PER_WG : a.B;
+    static_assert(R == 1 || R == HK_B_PER_WG, "rows per workgroup");
+    const int b_lo = blockIdx.y * R;
+    const int b_hi = b_lo + R < a.B ? b_lo + R : a.B;
 
     // every load of the workgroup is issued before anything waits: the inputs of
     // its batch rows first (they are needed first), then the weights of both
@@ -139,82 +154,114 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     if (a.zero_words) {
         const int64_t n_wg = static_cast<int64_t>(gridDim.x) * gridDim.y;
         const int64_t wg = static_cast<int64_t>(blockIdx.y) * gridDim.x + blockIdx.x;
-        for (int64_t i = wg * HK_THREADS + tid; i < a.zero_count; i += n_wg * HK_THREADS) a.zero_words[i] = 0u;
+        // 16 bytes per store while whole quads remain, single words for the tail
+        uint4 *z4 = reinterpret_cast<uint4 *>(a.zero_words);
+        const int64_t n4 = sl_aligned_dev(a.zero_words, 16) ? a.zero_count / 4 : 0;
+        for (int64_t i = wg * HK_THREADS + tid; i < n4; i += n_wg * HK_THREADS) z4[i] = make_uint4(0u, 0u, 0u, 0u);
+        for (int64_t i = n4 * 4 + wg * HK_THREADS + tid; i < a.zero_count; i += n_wg * HK_THREADS) a.zero_words[i] = 0u;
     }
 
-#pragma unroll 1  // keeps the kernel small: it mostly runs on compute units that do not hold its code yet
-    for (int b = b_lo; b < b_hi; ++b) {
-        const int bi = b - b_lo;
-        const float x_cur = bi == 0 ? x0 : bi == 1 ? x1 : bi == 2 ? x2 : x3;
-        const int32_t row_b = bi == 0 ? row0 : bi == 1 ? row1 : bi == 2 ? row2 : row3;
-        if (tid < HK_DIN) xs[tid] = x_cur;
-        __syncthreads();
+    const float xrow[4] = {x0, x1, x2, x3};
+    const int32_t drow[4] = {row0, row1, row2, row3};
+    if (tid < HK_DIN) {
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) xs[rr][tid] = xrow[rr];
+    }
+    __syncthreads();
 
-        // first projection
-        {
-            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // first projection
+    {
+        float acc[R][8];
 #pragma unroll
-            for (int q = 0; q < S1::PASSES; ++q) {
-                const float xv = xs[r + S1::RPP * q];
+        for (int rr = 0; rr < R; ++rr)
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] = fmaf(xv, w1r[q][j], acc[j]);
+            for (int j = 0; j < 8; ++j) acc[rr][j] = 0.f;
+#pragma unroll
+        for (int q = 0; q < S1::PASSES; ++q) {
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+                const float xv = xs[rr][r + S1::RPP * q];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[rr][j] = fmaf(xv, w1r[q][j], acc[rr][j]);
             }
-            float4 *dst = reinterpret_cast<float4 *>(&red[r * D_HID + cg * 8]);
-            dst[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-            dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            float4 *dst = reinterpret_cast<float4 *>(&red[rr * TABLE + r * D_HID + cg * 8]);
+            dst[0] = make_float4(acc[rr][0], acc[rr][1], acc[rr][2], acc[rr][3]);
+            dst[1] = make_float4(acc[rr][4], acc[rr][5], acc[rr][6], acc[rr][7]);
+        }
+    }
+    __syncthreads();
+    float v1[R];
+    fold_columns<D_HID, R>(red, sub, v1);
+    if (tid < D_HID) {
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            float v = round_to<T>(v1[rr]);
+            if (sd.b1) v = round_to<T>(v + bias1);
+            if constexpr (NL == 2) {
+                v = round_to<T>(silu_f32(v));
+                if (a.residue) v = round_to<T>(v + xs[rr][tid]);
+                hidl[rr][tid] = v;
+            } else {
+                if (a.residue) v = round_to<T>(v + xs[rr][tid]);
+            }
+            v1[rr] = v;
+        }
+    }
+    float pre[R];  // the pre-activations whose signs are the code: lanes tid < nbits
+    if constexpr (NL == 1) {
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) pre[rr] = v1[rr];
+    } else {
+        __syncthreads();
+        // second projection
+        {
+            float acc[R][8];
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[rr][j] = 0.f;
+#pragma unroll
+            for (int q = 0; q < P2; ++q) {
+#pragma unroll
+                for (int rr = 0; rr < R; ++rr) {
+                    const float hv = hidl[rr][r2 + R2 * q];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[rr][j] = fmaf(hv, w2r[q][j], acc[rr][j]);
+                }
+            }
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+                float4 *dst = reinterpret_cast<float4 *>(&red[rr * TABLE + r2 * HK_NBITS + cg2 * 8]);
+                dst[0] = make_float4(acc[rr][0], acc[rr][1], acc[rr][2], acc[rr][3]);
+                dst[1] = make_float4(acc[rr][4], acc[rr][5], acc[rr][6], acc[rr][7]);
+            }
         }
         __syncthreads();
-        float v1 = fold_columns<D_HID>(red, sub);
-        if (tid < D_HID) {
-            v1 = round_to<T>(v1);
-            if (sd.b1) v1 = round_to<T>(v1 + bias1);
-            if constexpr (NL == 2) {
-                v1 = round_to<T>(silu_f32(v1));
-                if (a.residue) v1 = round_to<T>(v1 + xs[tid]);
-                hidl[tid] = v1;
-            } else {
-                if (a.residue) v1 = round_to<T>(v1 + xs[tid]);
+        fold_columns<HK_NBITS, R>(red, sub, pre);
+        if (tid < HK_NBITS) {
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+                float v = round_to<T>(pre[rr]);
+                if (sd.b2) v = round_to<T>(v + bias2);
+                if (a.residue) v = round_to<T>(v + hidl[rr][tid]);
+                pre[rr] = v;
             }
         }
-        uint32_t *code_dst = sd.codes + static_cast<int64_t>(b) * sd.code_stride_b +
-                             static_cast<int64_t>(sd.code_row ? row_b : 0) * sd.code_stride_n +
-                             static_cast<int64_t>(h) * sd.code_stride_h;
-        if constexpr (NL == 1) {
-            // waves 0 .. D_HID/64-1 hold the pre-activations: 64 sign bits per wave
-            const uint64_t mask = __ballot(tid < D_HID && v1 > 0.f);
-            if (tid < D_HID && (tid & 63) == 0) {
-                code_dst[(tid >> 6) * 2] = static_cast<uint32_t>(mask);
-                code_dst[(tid >> 6) * 2 + 1] = static_cast<uint32_t>(mask >> 32);
-            }
-            __syncthreads();
-        } else {
-            __syncthreads();
-            // second projection
-            {
-                float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    }
+    // sign bits: the waves that hold the nbits pre-activations ballot 64 bits each
+    const int nbits = NL == 1 ? D_HID : HK_NBITS;
 #pragma unroll
-                for (int q = 0; q < P2; ++q) {
-                    const float hv = hidl[r2 + R2 * q];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) acc[j] = fmaf(hv, w2r[q][j], acc[j]);
-                }
-                float4 *dst = reinterpret_cast<float4 *>(&red[r2 * HK_NBITS + cg2 * 8]);
-                dst[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-                dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
-            }
-            __syncthreads();
-            float v2 = fold_columns<HK_NBITS>(red, sub);
-            if (tid < HK_NBITS) {
-                v2 = round_to<T>(v2);
-                if (sd.b2) v2 = round_to<T>(v2 + bias2);
-                if (a.residue) v2 = round_to<T>(v2 + hidl[tid]);
-            }
-            const uint64_t mask = __ballot(tid < HK_NBITS && v2 > 0.f);
-            if (tid < HK_NBITS && (tid & 63) == 0) {
-                code_dst[(tid >> 6) * 2] = static_cast<uint32_t>(mask);
-                code_dst[(tid >> 6) * 2 + 1] = static_cast<uint32_t>(mask >> 32);
-            }
-            __syncthreads();
+    for (int rr = 0; rr < R; ++rr) {
+        const uint64_t mask = __ballot(tid < nbits && pre[rr] > 0.f);
+        if (tid < nbits && (tid & 63) == 0 && b_lo + rr < b_hi) {
+            uint32_t *code_dst = sd.codes + static_cast<int64_t>(b_lo + rr) * sd.code_stride_b +
+                                 static_cast<int64_t>(sd.code_row ? drow[rr] : 0) * sd.code_stride_n +
+                                 static_cast<int64_t>(h) * sd.code_stride_h;
+            code_dst[(tid >> 6) * 2] = static_cast<uint32_t>(mask);
+            code_dst[(tid >> 6) * 2 + 1] = static_cast<uint32_t>(mask >> 32);
         }
     }
 
@@ -229,8 +276,12 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
 
 template <typename T, int NL, int D_HID>
 int launch3(const hash_args &a, int Htot, hipStream_t s) {
-    const dim3 grid(Htot, (a.B + HK_B_PER_WG - 1) / HK_B_PER_WG);
-    hash_kernel<T, NL, D_HID><<<grid, dim3(HK_THREADS), 0, s>>>(a);
+    if (a.B == 1) {
+        hash_kernel<T, NL, D_HID, 1><<<dim3(Htot, 1), dim3(HK_THREADS), 0, s>>>(a);
+    } else {
+        const dim3 grid(Htot, (a.B + HK_B_PER_WG - 1) / HK_B_PER_WG);
+        hash_kernel<T, NL, D_HID, HK_B_PER_WG><<<grid, dim3(HK_THREADS), 0, s>>>(a);
+    }
     return sl_check_launch();
 }
 

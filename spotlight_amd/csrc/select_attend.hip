@@ -69,6 +69,7 @@ __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args s
 template <typename T, int G>
 int launch_ng(const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
     if (sa.hist_groups == 16) select_attend_kernel<T, G, 16><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
+    else if (sa.hist_groups == 8) select_attend_kernel<T, G, 8><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
     else select_attend_kernel<T, G, 4><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
     return sl_check_launch();
 }
@@ -90,7 +91,7 @@ bool sl_select_attend_supported(const select_args &sa, const attn_args &aa) {
     const int64_t blocks = (sa.n + SA_BLOCK - 1) / SA_BLOCK;
     return (G == 1 || G == 2 || G == 4) && blocks <= SA_MAX_BLOCKS && blocks <= sa.hist_groups &&
            sa.hist_span == SA_BLOCK && sa.n_bins <= SA_THREADS * SA_MAX_BPT &&
-           (sa.hist_groups == 4 || sa.hist_groups == 16) && sa.stride_n == 1 && sa.stride_b % 8 == 0 &&
+           (sa.hist_groups == 4 || sa.hist_groups == 8 || sa.hist_groups == 16) && sa.stride_n == 1 && sa.stride_b % 8 == 0 &&
            sa.stride_h % 8 == 0 && sa.stride_h >= (sa.n + 7) / 8 * 8 && sl_aligned(sa.score, 16) && aa.B <= 65535;
 }
 

@@ -8,7 +8,7 @@ constexpr int TK_MAX_BINS = 4608;
 struct select_args {
     const int16_t *score;     // element (b, t, h) at b*stride_b + t*stride_n + h*stride_h
     uint32_t *hist;           // [B, KH, hist_groups, n_bins]: the copies are summed
-    int hist_groups;          // 4, 16 or 32
+    int hist_groups;          // 4, 8, 16 or 32
     int hist_span;            // token t is counted into copy (t / hist_span) % hist_groups
     int32_t *thr_need;        // [B, KH, 2] scratch: threshold bin, tokens to take from it
     uint32_t *block_cnt;      // [B, KH, n_blocks] scratch: (above | equal << 16) per token block

@@ -179,7 +179,7 @@ __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args 
 static int g_hist_copies = 0;  // sl_tune("hist_copies", 4 | 16); 0 = by cache length
 
 int sl_select_tune(const char *key, int value) {
-    if (!strcmp(key, "hist_copies") && (value == 0 || value == 4 || value == 16 || value == 32)) { g_hist_copies = value; return SL_OK; }
+    if (!strcmp(key, "hist_copies") && (value == 0 || value == 4 || value == 8 || value == 16 || value == 32)) { g_hist_copies = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
 
@@ -188,10 +188,10 @@ int sl_select_hist_groups(int64_t n) {
     // Copies of every histogram bin: they spread the same-bin adds of the many
     // scorer workgroups of one (b, kv head) over as many addresses, and copy c
     // counts the tokens of span c, which is what lets one launch select (see the
-    // top of this file).  16 for long caches, 4 for short ones (the copies must be
-    // cleared and read every step), 32 beyond 16 spans so that the single-launch
+    // top of this file).  16 for long caches, 4 or 8 for short ones (the copies must
+    // be cleared and read every step), 32 beyond 16 spans so that the single-launch
     // selection reaches 256k tokens.
-    return n > 16 * TK_BLOCK ? 32 : n > 4 * 4096 ? 16 : 4;
+    return n > 16 * TK_BLOCK ? 32 : n > 8 * 4096 ? 16 : n > 4 * 4096 ? 8 : 4;
 }
 
 int64_t sl_select_hist_span(int64_t n) {
@@ -234,7 +234,7 @@ int sl_select_launch(const select_args &a, hipStream_t s) {
                         a.stride_h >= (a.n + 7) / 8 * 8;
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(bh));
     const bool small = a.n_bins <= TK_THREADS;  // one bin per lane: the common case (G * nbits <= 1023)
-    SL_REQUIRE(a.hist_groups == 4 || a.hist_groups == 16 || a.hist_groups == 32, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(a.hist_groups == 4 || a.hist_groups == 8 || a.hist_groups == 16 || a.hist_groups == 32, SL_ERR_UNSUPPORTED);
     SL_REQUIRE(a.hist_span > 0 && TK_BLOCK % a.hist_span == 0, SL_ERR_UNSUPPORTED);
     // one launch while the copies do not wrap around (and one bin per lane, contiguous scores)
     const bool ordered = a.n <= static_cast<int64_t>(a.hist_groups) * a.hist_span;
@@ -251,6 +251,7 @@ int sl_select_launch(const select_args &a, hipStream_t s) {
     do {                                                          \
         if (a.hist_groups == 32) SL_SELECT_LAUNCH(CONTIG, BPT, 32); \
         else if (a.hist_groups == 16) SL_SELECT_LAUNCH(CONTIG, BPT, 16); \
+        else if (a.hist_groups == 8) SL_SELECT_LAUNCH(CONTIG, BPT, 8);   \
         else SL_SELECT_LAUNCH(CONTIG, BPT, 4);                    \
     } while (0)
     if (contig) {
