@@ -67,7 +67,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS) + ["c5"])
     ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch heuristic passed to sl_tune (e.g. attn_target_wgs=128)")
@@ -87,6 +87,8 @@ def main():
 
     from spotlight_amd import _lib, decode, kernel
 
+    if args.config == "c5":
+        return run_e2e(args)
     for kv in args.tune:
         key, val = kv.split("=")
         _lib.check(_lib.load().sl_tune(key.encode(), int(val)), f"sl_tune({kv})")
@@ -264,6 +266,186 @@ def main():
         "kernels": kernels, "roofline": roofline, "cpu_baseline": cpu_baseline,
     }
     print(json.dumps(out), flush=True)
+
+
+def run_e2e(args):
+    """c5: a random-init Llama-3-8B (32 layers, hidden 4096, 32 q / 8 kv heads, MLP 14336,
+    vocab 128256, rope theta 5e5), batch 4, 32768-token prompt prefilled densely, then
+    greedy decoding with layers 0-1 dense and layers 2.. on the sparse step (k = 655,
+    MLP hash 128-256-128 per query head and per kv head).  One decoded token for the
+    whole batch and all layers is ONE captured HIP graph (positions and lengths live on
+    the device); `value` is decoded tokens per second over the timed replays."""
+    import torch
+    import torch.nn.functional as F
+
+    from spotlight_amd import decode, kernel
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    dt = torch.bfloat16
+    B, n0, QH, KH, d, hidden, inter, vocab, theta, k = 4, 32768, 32, 8, 128, 4096, 14336, 128256, 5e5, 655
+    L = args.layers or 32
+    steps = args.steps if args.steps is not None else 512
+    warmup = args.warmup if args.warmup is not None else 8
+    fix_layers = (0, 1)
+    n_cap = (n0 + steps + warmup + 16 + 7) // 8 * 8
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    cg = torch.Generator()
+    cg.manual_seed(0)
+    rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * 0.02).to(dt)
+    embed, lm_head = rnd(vocab, hidden), rnd(vocab, hidden)
+    layers = []
+    for li in range(L):
+        w = dict(wq=rnd(QH * d, hidden), wk=rnd(KH * d, hidden), wv=rnd(KH * d, hidden), wo=rnd(hidden, QH * d),
+                 wg=rnd(inter, hidden), wu=rnd(inter, hidden), wd=rnd(hidden, inter),
+                 n1=torch.ones(hidden, device=dev, dtype=dt), n2=torch.ones(hidden, device=dev, dtype=dt))
+        if li in fix_layers:
+            w["kc"] = torch.zeros((B, KH, n_cap, d), device=dev, dtype=dt)   # head-major: SDPA reads it in place
+            w["vc"] = torch.zeros((B, KH, n_cap, d), device=dev, dtype=dt)
+        else:
+            hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dt, dev, cg)
+            hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dt, dev, cg)
+            w["st"] = decode.LayerDecodeState(B, QH, KH, d, n_cap, k, hq, hk, dtype=dt, device=dev)
+        layers.append(w)
+    norm_f = torch.ones(hidden, device=dev, dtype=dt)
+    inv_freq = 1.0 / (theta ** (torch.arange(0, d, 2, device=dev, dtype=torch.float32) / d))
+
+    def rms(x, w):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).to(dt) * w
+
+    def rope(x, pos):   # x [..., t, H, d], pos [t] (device)
+        ang = pos.float()[:, None] * inv_freq[None, :]
+        emb = torch.cat((ang, ang), dim=-1)
+        cos, sin = emb.cos().to(dt)[:, None, :], emb.sin().to(dt)[:, None, :]
+        rot = torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
+        return x * cos + rot * sin
+
+    def mlp(w, h):
+        return (F.silu(h @ w["wg"].T) * (h @ w["wu"].T)) @ w["wd"].T
+
+    # ---- prefill: dense causal attention in every layer (the draft is not used there), one sequence at a time
+    t_pre = time.perf_counter()
+    pos0 = torch.arange(n0, device=dev)
+    first = torch.empty((B,), dtype=torch.int64, device=dev)
+    with torch.no_grad():
+        for b in range(B):
+            ids = torch.randint(0, vocab, (n0,), generator=g, device=dev)
+            x = embed[ids]                                                   # [n0, hidden]
+            for w in layers:
+                h = rms(x, w["n1"])
+                q = rope((h @ w["wq"].T).view(n0, QH, d), pos0)
+                kk = rope((h @ w["wk"].T).view(n0, KH, d), pos0)
+                vv = (h @ w["wv"].T).view(n0, KH, d)
+                o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], kk.transpose(0, 1)[None],
+                                                   vv.transpose(0, 1)[None], is_causal=True, enable_gqa=True)
+                x = x + o[0].transpose(0, 1).reshape(n0, QH * d) @ w["wo"].T
+                x = x + mlp(w, rms(x, w["n2"]))
+                if "st" in w:
+                    st = w["st"]
+                    st.keys[b, :n0] = kk
+                    st.vals[b, :n0] = vv
+                    kernel.cache_append(st.codes[b:b + 1], st.hash_k.hash_rows(kk[None]), start=0)
+                else:
+                    w["kc"][b, :, :n0] = kk.transpose(0, 1)
+                    w["vc"][b, :, :n0] = vv.transpose(0, 1)
+            first[b] = (rms(x[-1:], norm_f) @ lm_head.T).float().argmax(dim=-1)[0]
+            del x, h, q, kk, vv, o
+        for w in layers:
+            if "st" in w:
+                w["st"].seq_lens.fill_(n0)
+                w["st"].host_len = n0
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t_pre
+
+    # ---- one decoded token = one graph
+    tok = first.clone()
+    pos = torch.full((1,), n0, dtype=torch.int64, device=dev)
+    n_max = n_cap
+    col = torch.arange(n_cap, device=dev)
+
+    def step_body():
+        x = embed[tok]                                                       # [B, hidden]
+        for w in layers:
+            h = rms(x, w["n1"])
+            q = rope((h @ w["wq"].T).view(B, 1, QH, d), pos)[:, 0]
+            kk = rope((h @ w["wk"].T).view(B, 1, KH, d), pos)[:, 0]
+            vv = (h @ w["wv"].T).view(B, KH, d)
+            if "st" in w:
+                st = w["st"]
+                st.q_in.copy_(q)
+                st.k_in.copy_(kk)
+                st.v_in.copy_(vv)
+                st._launch(n_max)
+                o = st.out.reshape(B, QH * d)
+            else:
+                w["kc"].index_copy_(2, pos, kk[:, :, None])
+                w["vc"].index_copy_(2, pos, vv[:, :, None])
+                # dense decode attention as two batched GEMMs per kv head group (the G query heads of
+                # a kv head are the G rows of the left operand: no K/V expansion, K and V read once)
+                sc = torch.matmul(q.view(B, KH, QH // KH, d), w["kc"].transpose(2, 3)).float() * (d ** -0.5)
+                sc = sc.masked_fill((col > pos)[None, None, None, :], float("-inf"))
+                o = torch.matmul(torch.softmax(sc, dim=-1).to(dt), w["vc"]).reshape(B, QH * d)
+            x = x + o @ w["wo"].T
+            x = x + mlp(w, rms(x, w["n2"]))
+        tok.copy_((rms(x, norm_f) @ lm_head.T).float().argmax(dim=-1))
+        pos.add_(1)
+
+    with torch.no_grad():
+        step_body()                                                          # eager once (lazy initialisations)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step_body()
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        gpu_ms = e0.elapsed_time(e1)
+        # the sparse attention's share: a graph with only the sparse layers' launches
+        sparse = [w["st"] for w in layers if "st" in w]
+        ga = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(ga):
+            for st in sparse:
+                st._launch(n_max, _STAGES_NO_ADVANCE)
+        ga.replay()
+        torch.cuda.synchronize()
+        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a0.record()
+        for _ in range(32):
+            ga.replay()
+        a1.record()
+        torch.cuda.synchronize()
+        attn_ms = a0.elapsed_time(a1) / 32
+    ms_per_step = max(wall_ms, gpu_ms) / steps
+    lens = [int(w["st"].seq_lens[0]) for w in layers if "st" in w]
+    assert all(v == lens[0] for v in lens), "sparse layers disagree on the cache length"
+    out = {
+        "metric": "e2e greedy decode tokens/s (random-init Llama-3-8B, batch 4, 32k prompt)",
+        "value": round(B / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "c5: random-init Llama-3-8B end to end, batch 4, 32768-token dense prefill, greedy decode, "
+                               "layers 0-1 dense, k=655", "layers": L, "batch": B, "context": n0, "k": k,
+                   "graph": "one HIP graph per decoded token (all layers)"},
+        "prefill_s": round(prefill_s, 2), "cache_len_after": lens[0] if lens else None,
+        "sparse_attention_ms_per_step": round(attn_ms, 4),
+        "sparse_attention_us_per_layer": round(attn_ms * 1e3 / max(1, len(sparse)), 2),
+        "sparse_attention_share": round(attn_ms / ms_per_step, 4),
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(out), flush=True)
+
+
+_STAGES_NO_ADVANCE = 1 | 2 | 4 | 16     # hash, score, select, attention launched as stages: lengths do not advance
 
 
 STAGE_KERNEL = {"hash": "hash_kernel", "score": "hamming_kernel", "select": "select_fused_kernel",
