@@ -307,11 +307,12 @@ def test_decode_step_two_launch_tail_matches_oracle(env, B, QH, KH, n0, k, dtype
 
 
 def test_decode_many_blocks_and_long_cache(env):
-    """More than one 4096-token block per (b, kv head) in the fused tail; 8192-token
+    """More than one 4096-token block per (b, kv head) in the fused tail (4 and 8
+    histogram copies); 8192-token
     spans with 16 and with 32 histogram copies (single-launch selection); and the
     two-launch selector once the copies wrap around (beyond 256k tokens)."""
     decode, kernel = env
-    for n0, k in ((9000, 180), (70000, 300), (140000, 500), (270000, 64)):
+    for n0, k in ((9000, 180), (20000, 100), (70000, 300), (140000, 500), (270000, 64)):
         g = _gen(n0)
         st = _make_state(decode, g, 1, 8, 2, n0, (n0 + 64 + 7) // 8 * 8, k, torch.bfloat16)
         for step in range(2):
