@@ -6,6 +6,12 @@ struct attn_args {
     const void *q;          // [B, QH, 128]
     const void *keys, *vals;
     const int32_t *idx;     // [B, KH, k] row numbers, negative = skip
+    // optional deferred fetch (LRU misses): fetch[b,h,i] >= 0 names the row of the SOURCE store
+    // that row idx[b,h,i] of keys / vals has to be filled from; the kernel reads the source
+    // row, uses it, and writes it to keys / vals (which are then written to)
+    const int32_t *fetch;
+    const void *src_keys, *src_vals;
+    int64_t src_stride_b, src_stride_n, src_stride_h;
     void *out;              // [B, QH, 128]
     float *part;            // workspace: [B*KH][S][G][130] partial (acc, m, l)
     uint32_t *counter;      // workspace: [B*KH] arrival tickets, left at zero

@@ -22,18 +22,23 @@ constexpr int AT_MAX_ROWS = 1024;    // rows per run (LDS row-number buffer)
 // the only part that has to stay zero between calls.
 constexpr size_t AT_COUNTER_BYTES = 64 * 1024;
 
-template <typename T, int G, int NW>
+template <typename T, int G, int NW, bool FETCH>
 __global__ __launch_bounds__(NW * 64) void sparse_attn_kernel(attn_args a) {
     constexpr int AT_THREADS = NW * 64;
     __shared__ int s_row[AT_MAX_ROWS];
+    __shared__ int s_src[FETCH ? AT_MAX_ROWS : 1];
     __shared__ attn_shared<G, NW> sh;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int r_lo = split * a.rows;
     const int r_hi = r_lo + a.rows < a.k ? r_lo + a.rows : a.k;
     const int32_t *idx = a.idx + (static_cast<int64_t>(b) * a.KH + h) * a.k;
     for (int i = threadIdx.x; i < a.rows; i += AT_THREADS) s_row[i] = r_lo + i < r_hi ? idx[r_lo + i] : -1;
+    if constexpr (FETCH) {
+        const int32_t *fetch = a.fetch + (static_cast<int64_t>(b) * a.KH + h) * a.k;
+        for (int i = threadIdx.x; i < a.rows; i += AT_THREADS) s_src[i] = r_lo + i < r_hi ? fetch[r_lo + i] : -1;
+    }
     __syncthreads();
-    attend_rows_and_merge<T, G, NW>(a, b, h, split, gridDim.x, s_row, a.rows, sh);
+    attend_rows_and_merge<T, G, NW, FETCH>(a, b, h, split, gridDim.x, s_row, a.rows, sh, s_src);
 }
 
 int g_attn_wide_rows = AT_WIDE_ROWS;  // sl_tune("attn_wide_rows", n)
@@ -41,8 +46,15 @@ int g_attn_wide_rows = AT_WIDE_ROWS;  // sl_tune("attn_wide_rows", n)
 template <typename T, int G>
 int launch(const attn_args &a, hipStream_t s) {
     const int S = (a.k + a.rows - 1) / a.rows;
-    if (a.rows >= g_attn_wide_rows) sparse_attn_kernel<T, G, 8><<<dim3(S, a.KH, a.B), dim3(512), 0, s>>>(a);
-    else sparse_attn_kernel<T, G, 4><<<dim3(S, a.KH, a.B), dim3(256), 0, s>>>(a);
+    const dim3 grid(S, a.KH, a.B);
+    const bool wide = a.rows >= g_attn_wide_rows;
+    if (a.fetch) {
+        if (wide) sparse_attn_kernel<T, G, 8, true><<<grid, dim3(512), 0, s>>>(a);
+        else sparse_attn_kernel<T, G, 4, true><<<grid, dim3(256), 0, s>>>(a);
+    } else {
+        if (wide) sparse_attn_kernel<T, G, 8, false><<<grid, dim3(512), 0, s>>>(a);
+        else sparse_attn_kernel<T, G, 4, false><<<grid, dim3(256), 0, s>>>(a);
+    }
     return sl_check_launch();
 }
 
@@ -104,6 +116,7 @@ int sl_attn_launch(attn_args a, void *ws, size_t ws_bytes, hipStream_t s) {
     const int rc = sl_attn_prepare(a, ws, ws_bytes);
     if (rc != SL_OK) return rc;
     if (a.rows <= 0) a.rows = pick_rows(a.B, a.KH, a.k);
+    if (a.fetch) SL_REQUIRE(a.src_keys && a.src_vals, SL_ERR_NULL);
     SL_REQUIRE(a.rows % AT_ITER_ROWS == 0 && a.rows <= AT_MAX_ROWS, SL_ERR_UNSUPPORTED);
     SL_REQUIRE((a.k + a.rows - 1) / a.rows <= AT_MAX_SPLITS, SL_ERR_UNSUPPORTED);  // k <= 16384
     switch (a.dtype) {

@@ -75,6 +75,15 @@ template <typename T> __device__ __forceinline__ slice8<T> load_slice8(const T *
     return s;
 }
 
+template <typename T> __device__ __forceinline__ void store_slice8(T *p, const slice8<T> &s) {
+    if constexpr (sizeof(T) == 4) {
+        reinterpret_cast<float4 *>(p)[0] = s.a;
+        reinterpret_cast<float4 *>(p)[1] = s.b;
+    } else {
+        *reinterpret_cast<uint4 *>(p) = s.w;
+    }
+}
+
 typedef __bf16 sl_bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 sl_f16x2 __attribute__((ext_vector_type(2)));
 
@@ -109,6 +118,11 @@ template <typename T> __device__ __forceinline__ pair_raw<T> load_pair(const T *
     if constexpr (sizeof(T) == 4) r.v = *reinterpret_cast<const float2 *>(p);
     else r.w = *reinterpret_cast<const uint32_t *>(p);
     return r;
+}
+
+template <typename T> __device__ __forceinline__ void store_pair(T *p, const pair_raw<T> &r) {
+    if constexpr (sizeof(T) == 4) *reinterpret_cast<float2 *>(p) = r.v;
+    else *reinterpret_cast<uint32_t *>(p) = r.w;
 }
 
 template <typename T> __device__ __forceinline__ void unpack_pair(const pair_raw<T> &r, float &lo, float &hi) {
@@ -171,10 +185,14 @@ template <int U> __device__ __forceinline__ float head_max(float v) {
 
 // Attends over the rows listed in s_row[0 .. n_rows) (LDS; negative = skipped), as
 // run `split` of `S` runs of the (b, kv head).  Every lane of the workgroup must
-// call it; the caller has already synchronised the writes to s_row.
-template <typename T, int G, int NW>
+// call it; the caller has already synchronised the writes to s_row.  With FETCH,
+// s_src[i] >= 0 names a row of the source store that row s_row[i] is to be filled
+// from: the kernel reads that row instead, and writes the K slices / V pairs it
+// loaded to row s_row[i] of keys / vals after it has used them.
+template <typename T, int G, int NW, bool FETCH = false>
 __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b, int h, int split, int S,
-                                                      const int *s_row, int n_rows, attn_shared<G, NW> &sh) {
+                                                      const int *s_row, int n_rows, attn_shared<G, NW> &sh,
+                                                      const int *s_src = nullptr) {
     using SH = attn_shared<G, NW>;
     constexpr int NT = NW * 64, NLG = SH::NLG, GP = SH::GP, U = SH::U, CH = SH::CH, RW = SH::RW;
     const int tid = threadIdx.x;
@@ -192,6 +210,13 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
                   static_cast<int64_t>(h) * a.kv_stride_h + sub * 8;
     const T *vb = static_cast<const T *>(a.vals) + static_cast<int64_t>(b) * a.kv_stride_b +
                   static_cast<int64_t>(h) * a.kv_stride_h + lane * 2;
+    const T *skb = nullptr, *svb = nullptr;
+    if constexpr (FETCH) {
+        skb = static_cast<const T *>(a.src_keys) + static_cast<int64_t>(b) * a.src_stride_b +
+              static_cast<int64_t>(h) * a.src_stride_h + sub * 8;
+        svb = static_cast<const T *>(a.src_vals) + static_cast<int64_t>(b) * a.src_stride_b +
+              static_cast<int64_t>(h) * a.src_stride_h + lane * 2;
+    }
 
     float m_run[GP], lsum[G], acc[G][2];
 #pragma unroll
@@ -203,23 +228,33 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         // every load of the chunk first: U key slices for the score phase, RW value
         // pairs for the accumulation phase (an absent or skipped row re-reads row 0
         // and gets probability 0): no branch sits between the loads
-        int row[U];
+        int row[U], src[U];
         slice8<T> ks[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int ri = base + u * NLG + rslot;
             row[u] = ri < n_rows ? s_row[ri] : -1;
+            src[u] = FETCH && ri < n_rows && row[u] >= 0 ? s_src[ri] : -1;
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-            ks[u] = load_slice8<T>(kb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n);
+        for (int u = 0; u < U; ++u) {
+            const T *p = kb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n;
+            if constexpr (FETCH) p = src[u] >= 0 ? skb + static_cast<int64_t>(src[u]) * a.src_stride_n : p;
+            ks[u] = load_slice8<T>(p);
+        }
         pair_raw<T> vs[RW];
+        int vrow[RW], vsrc[RW];
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
             const int ri = base + wave + NW * j;
             int r = ri < n_rows ? s_row[ri] : -1;
+            int sr = FETCH && ri < n_rows && r >= 0 ? s_src[ri] : -1;
+            vrow[j] = __builtin_amdgcn_readfirstlane(r);
+            vsrc[j] = __builtin_amdgcn_readfirstlane(sr);
             r = __builtin_amdgcn_readfirstlane(r >= 0 ? r : 0);  // the same row for the whole wave
-            vs[j] = load_pair<T>(vb + static_cast<int64_t>(r) * a.kv_stride_n);
+            const T *p = vb + static_cast<int64_t>(r) * a.kv_stride_n;
+            if constexpr (FETCH) p = vsrc[j] >= 0 ? svb + static_cast<int64_t>(vsrc[j]) * a.src_stride_n : p;
+            vs[j] = load_pair<T>(p);
         }
 
         // scores: partial dot products of this lane's slice, then the butterfly
@@ -230,6 +265,12 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             part[i] = g < G ? dot_slice8<T>(qs[g < G ? g : 0], ks[u]) : 0.f;
         }
         float s = row16_transpose_sum(part, sub) * a.scale;
+        if constexpr (FETCH) {
+            // the fetched K slices have been used (and therefore waited for): put them in their rows
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (src[u] >= 0) store_slice8<T>(const_cast<T *>(kb) + static_cast<int64_t>(row[u]) * a.kv_stride_n, ks[u]);
+        }
         int my_row = row[0];
 #pragma unroll
         for (int u = 1; u < U; ++u) my_row = u_l == u ? row[u] : my_row;
@@ -278,6 +319,11 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
                 acc[g][0] = fmaf(pg, v0, acc[g][0]);
                 acc[g][1] = fmaf(pg, v1, acc[g][1]);
             }
+        }
+        if constexpr (FETCH) {
+#pragma unroll
+            for (int j = 0; j < RW; ++j)
+                if (vsrc[j] >= 0) store_pair<T>(const_cast<T *>(vb) + static_cast<int64_t>(vrow[j]) * a.kv_stride_n, vs[j]);
         }
         if (base + CH < n_rows) __syncthreads();  // the next chunk rewrites wmax and p
     }

@@ -50,7 +50,7 @@ constexpr int LRU_CP = 4;  // 16-byte chunks of K and of V a lane keeps in fligh
     _Pragma("unroll") for (int u = 0; u < LRU_CP; ++u) {                                           \
         const int e = (E0) + u * LRU_THREADS + tid;                                                \
         const int ec = e < n_chunks ? e : 0;                                                       \
-        const int j = ec / CH, c = ec % CH;                                                        \
+        const int j = j_lo + ec / CH, c = ec % CH;                                                 \
         const int64_t src = (static_cast<int64_t>(s_miss_tok[j]) * a.KH + h) * CH + c;             \
         dsts[u] = e < n_chunks ? s_victim[j] * CH + c : -1;                                        \
         kbuf[u] = *reinterpret_cast<const u32x4 *>(kf + src);                                                                         \
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
     __shared__ uint32_t s_hist[256];
     __shared__ uint32_t s_wave[LRU_THREADS / 64 + 1];
     __shared__ uint32_t s_digit, s_remaining;
-    __shared__ int s_new_in;
+    __shared__ int s_new_in, s_new_pos;
 
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.KH, h = blockIdx.x % a.KH;
@@ -84,11 +84,12 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
     int32_t *ts = a.token_slot + bh * a.map_cap;
     const int32_t *idx = a.idx + bh * k;
     int32_t *so = a.slots_out + bh * k;
+    int32_t *fo = a.fetch_out ? a.fetch_out + bh * k : nullptr;
     const uint32_t t = a.stamp + (a.stamp_dev ? a.stamp_dev[0] : 0u);
     const int new_tok = a.new_token ? a.new_token[b] : -1;
 
     for (int s = tid; s < C; s += LRU_THREADS) s_flag[s] = 0;
-    if (tid == 0) s_new_in = 0;
+    if (tid == 0) { s_new_in = 0; s_new_pos = -1; }
     __syncthreads();
 
     // wanted items 0..k-1 = idx, item k = the new token unless idx already holds it
@@ -116,13 +117,13 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
                 if (slot[j] >= 0) {
                     s_flag[slot[j]] = 1;
                     ss[slot[j]] = t;
-                    if (i < k) so[i] = slot[j];
+                    if (i < k) { so[i] = slot[j]; if (fo) fo[i] = -1; }
                 } else {
                     ++n_miss;
                 }
             } else {
                 tok[j] = -1;
-                if (i < k) so[i] = -1;
+                if (i < k) { so[i] = -1; if (fo) fo[i] = -1; }
             }
         }
     }
@@ -137,6 +138,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
             if (tok[j] >= 0 && slot[j] < 0) {
                 s_miss_tok[pos] = tok[j];
                 s_miss_item[pos] = tid * IPT + j;
+                if (tid * IPT + j >= k) s_new_pos = static_cast<int>(pos);  // the new token, not among the selected
                 ++pos;
             }
     }
@@ -234,7 +236,10 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
         const uint4 *vf = static_cast<const uint4 *>(a.vals) + static_cast<int64_t>(b) * a.kv_stride_b * es / 16;
         uint4 *kr = static_cast<uint4 *>(a.k_res) + bh * C * CH;
         uint4 *vr = static_cast<uint4 *>(a.v_res) + bh * C * CH;
-        const int n_chunks = M * CH;
+        // with fetch_out the consumer fetches the selected misses; only the new token's
+        // row (when it is not among the selected) is copied here
+        const int j_lo = fo ? (s_new_pos >= 0 ? s_new_pos : 0) : 0;
+        const int n_chunks = fo ? (s_new_pos >= 0 ? CH : 0) : M * CH;
         // (a native vector type: arrays of the HIP uint4 struct were not kept in registers here)
         typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
         u32x4 kbuf[LRU_CP], vbuf[LRU_CP];
@@ -253,7 +258,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
             st[s] = tk;
             ss[s] = t;
             const int item = s_miss_item[j];
-            if (item < k) so[item] = s;
+            if (item < k) { so[item] = s; if (fo) fo[item] = tk; }
         }
         LRU_RETIRE()
         for (int e0 = LRU_CP * LRU_THREADS; e0 < n_chunks; e0 += LRU_CP * LRU_THREADS) {

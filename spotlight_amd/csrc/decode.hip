@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, ui
 int g_fuse_select_attend = 1;  // sl_tune("fuse_select_attend", 0 | 1 | 2): never, by shape, whenever possible
 
 struct ws_layout {
-    size_t q_code, select, score, attn, total;
+    size_t q_code, select, score, lru_fetch, attn, total;
 };
 
 ws_layout layout(const sl_decode_params &p) {
@@ -44,6 +44,7 @@ ws_layout layout(const sl_decode_params &p) {
     L.q_code = off; off += sl_align_up(sizeof(uint32_t) * p.B * p.QH * W, 256);
     L.select = off; off += sl_select_ws_bytes(p.B, p.KH, static_cast<int>(G * p.nbits + 1), p.n_cap);
     L.score = off;  off += sl_align_up(sizeof(int16_t) * p.B * p.KH * static_cast<size_t>(p.n_cap), 256);
+    L.lru_fetch = off; off += p.lru_C > 0 ? sl_align_up(sizeof(int32_t) * p.B * p.KH * static_cast<size_t>(p.k), 256) : 0;
     L.attn = off;   off += sl_attn_ws_bytes(p.B, p.QH, p.KH, p.k);
     L.total = off;
     return L;
@@ -208,6 +209,12 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         la.slots_out = p.slots_out; la.stats = p.lru_stats; la.stamp_dev = p.step_counter; la.stamp = 1;
         la.dtype = p.dtype; la.B = p.B; la.KH = p.KH; la.d = p.d; la.k = p.k; la.C = p.lru_C;
         la.map_cap = p.lru_map_cap; la.kv_stride_b = p.n_cap * p.KH * p.d;
+        // When the attention follows in the same call, it fetches the rows of the selected
+        // misses from the full store itself (it has to read them anyway) and drops them
+        // into their slots: the table update then copies no rows but the new token's.
+        const bool defer = (stages & SL_STAGE_LRU) && (stages & SL_STAGE_ATTN);
+        int32_t *fetch = reinterpret_cast<int32_t *>(ws + L.lru_fetch);
+        la.fetch_out = defer ? fetch : nullptr;
         if (stages & SL_STAGE_LRU) {
             rc = sl_lru_launch(la, s);
             if (rc != SL_OK) return rc;
@@ -216,6 +223,11 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         aa.kv_stride_b = static_cast<int64_t>(p.KH) * p.lru_C * p.d;
         aa.kv_stride_h = static_cast<int64_t>(p.lru_C) * p.d;
         aa.kv_stride_n = p.d;
+        if (defer) {
+            aa.fetch = fetch; aa.src_keys = p.keys; aa.src_vals = p.vals;
+            aa.src_stride_b = p.n_cap * p.KH * p.d; aa.src_stride_n = static_cast<int64_t>(p.KH) * p.d;
+            aa.src_stride_h = p.d;
+        }
     }
     if (!(stages & SL_STAGE_ATTN)) return SL_OK;
     return sl_attn_launch(aa, ws + L.attn, L.total - L.attn, s);

@@ -14,6 +14,9 @@ struct lru_args {
     const void *keys, *vals;   // full store [B, L, KH, d]
     void *k_res, *v_res;       // resident rows [B, KH, C, d]
     int32_t *slots_out;        // [B, KH, k]
+    int32_t *fetch_out;        // optional [B, KH, k]: when given, the rows of the selected misses are NOT
+                               // copied by this launch; entry i receives the token whose row the consumer
+                               // has to fetch from the full store into slot slots_out[i] (-1: resident)
     uint32_t *stats;           // [B, KH, 2] or null
     const uint32_t *stamp_dev; // optional device word added to `stamp`
     uint32_t stamp;
