@@ -131,11 +131,13 @@ def test_decode_ragged_batch(env):
         assert np.abs(out[b:b + 1] - want).max() <= 1e-5
 
 
-def test_decode_graph_replay_equals_eager(env):
-    """A captured step replayed while the cache grows gives what eager steps give."""
+@pytest.mark.parametrize("lru", [0, 64])
+def test_decode_graph_replay_equals_eager(env, lru):
+    """A captured step replayed while the cache grows gives what eager steps give
+    (also with the LRU table, whose misses the attention launch fetches)."""
     decode, kernel = env
     dtype = torch.bfloat16
-    states = [_make_state(decode, _gen(90), 2, 32, 8, 500, 640, 30, dtype) for _ in range(2)]
+    states = [_make_state(decode, _gen(90), 2, 32, 8, 500, 640, 30, dtype, lru=lru) for _ in range(2)]
     eager, graphed = states
     graphed.capture(steps_ahead=8)
     g = _gen(91)
@@ -150,6 +152,9 @@ def test_decode_graph_replay_equals_eager(env):
         assert torch.equal(eager.idx, graphed.idx), step
         assert torch.equal(a, b), step
         assert torch.equal(eager.seq_lens, graphed.seq_lens)
+        if lru:
+            assert torch.equal(eager.slot_token, graphed.slot_token) and torch.equal(eager.k_res, graphed.k_res)
+            assert torch.equal(eager.v_res, graphed.v_res)
     with pytest.raises(RuntimeError):
         for _ in range(5):
             graphed.replay()
