@@ -41,14 +41,8 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     const int b = blockIdx.y;
     const int KH = a.KH;
     const int G = G_T > 0 ? G_T : a.G;
-    int64_t n_b = a.n;
-    if (a.seq_lens) {
-        const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
-        n_b = l < n_b ? l : n_b;
-    }
     const int tok_per_pass = HS_THREADS / KH;
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * tok_per_pass * HS_U;
-    if (t0 >= n_b) return;
 
     const int tid = threadIdx.x;
     const int h = tid % KH;
@@ -62,7 +56,8 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
 
     // the query codes and the HS_U records of the lane are independent loads: all
     // are issued before the first wait.  Record loads are unconditional (rows past
-    // the end re-read the last row and are discarded below): no branch sits between them
+    // the bound a.n re-read the last row; rows past the sequence length are
+    // discarded below): no branch sits between them
     const uint32_t *qb = a.q_code + static_cast<int64_t>(b) * a.q_stride_b;
     uint32_t qreg[(G_T > 0 ? G_T : 1)][W];
     if constexpr (G_T > 0) {
@@ -74,14 +69,22 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     }
     const uint32_t *kb = a.k_code + static_cast<int64_t>(b) * a.k_stride_b;
     uint32_t kreg[HS_U][W];
-    bool valid[HS_U];
 #pragma unroll
     for (int u = 0; u < HS_U; ++u) {
         const int64_t t = t0 + static_cast<int64_t>(u) * tok_per_pass + tl;
-        valid[u] = t < n_b;
-        const int64_t tc = valid[u] ? t : n_b - 1;
-        load_code<W>(kb + (tc * KH + h) * W, kreg[u]);
+        load_code<W>(kb + ((t < a.n ? t : a.n - 1) * KH + h) * W, kreg[u]);  // a.n rows exist whatever the length is
     }
+    // the sequence length is only needed from here on: it is read from memory, and
+    // nothing above had to wait for it
+    int64_t n_b = a.n;
+    if (a.seq_lens) {
+        const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
+        n_b = l < n_b ? l : n_b;
+    }
+    if (t0 >= n_b) return;
+    bool valid[HS_U];
+#pragma unroll
+    for (int u = 0; u < HS_U; ++u) valid[u] = t0 + static_cast<int64_t>(u) * tok_per_pass + tl < n_b;
     if constexpr (G_T == 0) {
         // q_lds[(h*G + g)*W + w]
         for (int e = tid; e < KH * G * W; e += HS_THREADS) {
