@@ -326,3 +326,38 @@ def test_decode_many_blocks_and_long_cache(env):
             vn = torch.randn(1, 2, 128, generator=g).to(torch.bfloat16)
             out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV))
             _check_step(kernel, st, q, kn, vn, out, n0 + step, torch.bfloat16)
+
+
+def _random_cases(count, seed):
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(count):
+        KH = rnd.choice([1, 2, 4, 8, 16])
+        G = rnd.choice([1, 2, 3, 4, 5, 8])
+        while KH * G > 64:
+            G = rnd.choice([1, 2, 4])
+        B = rnd.choice([1, 2, 3, 5])
+        n0 = rnd.choice([1, 7, 63, 64, 65, 255, 256, 257, 1000, 2047, 4095, 4096, 4097, 8191, 8200])
+        k = rnd.choice([1, 2, 17, 64, 100, 333, 600])
+        dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+        kind = rnd.choice(["mlp", "mlp", "linear"])
+        if kind == "linear" and G != 1:
+            kind = "mlp"               # the linear hash of the reference is per head, no grouped variant
+        cases.append((B, KH * G, KH, n0, k, dtype, kind))
+    return cases
+
+
+@pytest.mark.parametrize("B,QH,KH,n0,k,dtype,kind", _random_cases(24, 2024))
+def test_decode_step_random_shapes(env, B, QH, KH, n0, k, dtype, kind):
+    """Seeded sweep over head counts, group sizes, batch sizes, cache lengths around the
+    block / tile / span boundaries, budgets above and below the cache length."""
+    decode, kernel = env
+    g = _gen(QH * 131 + n0 + k)
+    st = _make_state(decode, g, B, QH, KH, n0, (n0 + 16 + 7) // 8 * 8, k, dtype, kind)
+    for step in range(2):
+        q = torch.randn(B, QH, 128, generator=g).to(dtype)
+        k_new = torch.randn(B, KH, 128, generator=g).to(dtype)
+        v_new = torch.randn(B, KH, 128, generator=g).to(dtype)
+        out = st.step(q.to(DEV), k_new.to(DEV), v_new.to(DEV))
+        _check_step(kernel, st, q, k_new, v_new, out, n0 + step, dtype)
