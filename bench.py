@@ -69,6 +69,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS) + ["c5"])
     ap.add_argument("--layers", type=int, default=None)
+    ap.add_argument("--batch", type=int, default=None, help="override the configuration's batch size (c1-c4)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch heuristic passed to sl_tune (e.g. attn_target_wgs=128)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -93,6 +94,9 @@ def main():
         key, val = kv.split("=")
         _lib.check(_lib.load().sl_tune(key.encode(), int(val)), f"sl_tune({kv})")
     c = dict(CONFIGS[args.config])
+    if args.batch:
+        c["B"] = args.batch
+        c["desc"] += f", batch overridden to {args.batch}"
     L = args.layers or c["layers"]
     steps = args.steps if args.steps is not None else (256 if args.config == "c3" else 1000)
     warmup = args.warmup if args.warmup is not None else 64

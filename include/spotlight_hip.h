@@ -49,6 +49,8 @@ int sl_version(void);
  * "fuse_select_attend": 1 (default) lets the decode step run selection and
  * attention as one launch when the shapes allow and every 4096-token block keeps
  * at most 128 rows on average, 2 whenever the shapes allow, 0 never;
+ * "hash_rows": batch rows one hash workgroup takes through the projections together
+ * (1, 2 or 4; 0 = by batch size, the default);
  * "attn_wide_rows": rows per run from which the attention launch uses 8 waves per
  * workgroup instead of 4 (default 128);
  * "hist_copies": copies of the score histogram (4, 8, 16 or 32; 0 = by cache

@@ -84,8 +84,8 @@ extern "C" int sl_version(void) { return 100; }
 extern "C" int sl_tune(const char *key, int value) {
     SL_REQUIRE(key, SL_ERR_NULL);
     if (!strcmp(key, "fuse_select_attend") && value >= 0 && value <= 2) { g_fuse_select_attend = value; return SL_OK; }
-    const int rc = sl_attn_tune(key, value);
-    return rc == SL_OK ? rc : sl_select_tune(key, value);
+    if (sl_attn_tune(key, value) == SL_OK || sl_select_tune(key, value) == SL_OK) return SL_OK;
+    return sl_hash_tune(key, value);
 }
 
 extern "C" int sl_host_device_pointer(void *host_ptr, void **device_ptr) {

@@ -27,3 +27,4 @@ struct hash_args {
 };
 
 int sl_hash_launch(hash_args a, hipStream_t s);
+int sl_hash_tune(const char *key, int value);

@@ -24,6 +24,8 @@
 // (after the matmul, after the bias add, after SiLU, after the residual add).
 #include "hash.h"
 
+#include <string.h>
+
 namespace {
 
 constexpr int HK_THREADS = 512;
@@ -97,7 +99,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     const int side_i = (a.n_sides > 1 && hh >= a.side[0].H) ? 1 : 0;
     const hash_side &sd = a.side[side_i];
     const int h = hh - (side_i ? a.side[0].H : 0);
-    static_assert(R == 1 || R == HK_B_PER_WG, "rows per workgroup");
+    static_assert(R == 1 || R == 2 || R == HK_B_PER_WG, "rows per workgroup");
     const int b_lo = blockIdx.y * R;
     const int b_hi = b_lo + R < a.B ? b_lo + R : a.B;
 
@@ -274,14 +276,20 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     }
 }
 
+int g_hash_rows = 0;  // sl_tune("hash_rows", 0 | 1 | 2 | 4): batch rows per workgroup, 0 = by batch size
+
 template <typename T, int NL, int D_HID>
 int launch3(const hash_args &a, int Htot, hipStream_t s) {
-    if (a.B == 1) {
-        hash_kernel<T, NL, D_HID, 1><<<dim3(Htot, 1), dim3(HK_THREADS), 0, s>>>(a);
-    } else {
-        const dim3 grid(Htot, (a.B + HK_B_PER_WG - 1) / HK_B_PER_WG);
-        hash_kernel<T, NL, D_HID, HK_B_PER_WG><<<grid, dim3(HK_THREADS), 0, s>>>(a);
-    }
+    // Rows per workgroup: the fewest that still give every workgroup a compute unit of
+    // its own (256 of them); rows taken together share barriers and weights but each
+    // adds to the workgroup's critical path.
+    int rows = 1;
+    while (rows < HK_B_PER_WG && static_cast<int64_t>(Htot) * ((a.B + rows - 1) / rows) > 256) rows *= 2;
+    if (g_hash_rows && a.B > 1) rows = g_hash_rows;
+    const dim3 grid(Htot, (a.B + rows - 1) / rows);
+    if (rows == 1) hash_kernel<T, NL, D_HID, 1><<<grid, dim3(HK_THREADS), 0, s>>>(a);
+    else if (rows == 2) hash_kernel<T, NL, D_HID, 2><<<grid, dim3(HK_THREADS), 0, s>>>(a);
+    else hash_kernel<T, NL, D_HID, HK_B_PER_WG><<<grid, dim3(HK_THREADS), 0, s>>>(a);
     return sl_check_launch();
 }
 
@@ -303,6 +311,11 @@ int launch(const hash_args &a, int Htot, hipStream_t s) {
 
 }  // namespace
 
+int sl_hash_tune(const char *key, int value) {
+    if (!strcmp(key, "hash_rows") && (value == 0 || value == 1 || value == 2 || value == 4)) { g_hash_rows = value; return SL_OK; }
+    return SL_ERR_UNSUPPORTED;
+}
+
 int sl_hash_launch(hash_args a, hipStream_t s) {
     SL_REQUIRE(a.n_sides == 1 || a.n_sides == 2, SL_ERR_SHAPE);
     SL_REQUIRE(a.n_layers == 1 || a.n_layers == 2, SL_ERR_UNSUPPORTED);
@@ -311,7 +324,7 @@ int sl_hash_launch(hash_args a, hipStream_t s) {
     if (a.n_layers == 2) SL_REQUIRE(a.nbits == HK_NBITS, SL_ERR_UNSUPPORTED);
     if (a.n_layers == 1) SL_REQUIRE(a.nbits == a.d_hid, SL_ERR_SHAPE);
     if (a.residue) SL_REQUIRE(a.d_hid == a.d_in && (a.n_layers == 1 || a.nbits == a.d_hid), SL_ERR_SHAPE);
-    SL_REQUIRE((a.B + HK_B_PER_WG - 1) / HK_B_PER_WG <= 65535, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(a.B <= 65535, SL_ERR_UNSUPPORTED);
     int Htot = 0;
     for (int i = 0; i < a.n_sides; ++i) {
         const hash_side &sd = a.side[i];
