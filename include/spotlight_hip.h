@@ -262,7 +262,9 @@ int sl_decode_step(const sl_decode_params *p, void *stream);
 /* The same step restricted to a subset of its kernels, for profiling one
  * kernel at a time on real shapes.  Lengths and the step counter only advance
  * when every stage runs.  HASH also clears the score histogram, so SCORE
- * without a preceding HASH keeps adding to it. */
+ * without a preceding HASH keeps adding to it, and HASH leaves the step's row
+ * counts (seq_lens[b] + 1) in the workspace for the later stages: a subset
+ * without HASH works on the counts of the last HASH launch. */
 enum {
     SL_STAGE_HASH = 1, SL_STAGE_SCORE = 2, SL_STAGE_SELECT = 4, SL_STAGE_LRU = 8, SL_STAGE_ATTN = 16,
     SL_STAGE_ALL = 31

@@ -32,8 +32,11 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, ui
 
 int g_fuse_select_attend = 1;  // sl_tune("fuse_select_attend", 0 | 1 | 2): never, by shape, whenever possible
 
+// Only the attention tickets (head of `attn`) have to stay zero between calls.  Nothing in front of
+// them depends on k, so they keep their place when the caller lowers or raises k on a live workspace;
+// the one k-sized region comes last.
 struct ws_layout {
-    size_t q_code, select, score, lru_fetch, attn, total;
+    size_t q_code, attn, n_rows, select, score, lru_fetch, total;
 };
 
 ws_layout layout(const sl_decode_params &p) {
@@ -42,10 +45,11 @@ ws_layout layout(const sl_decode_params &p) {
     const size_t G = static_cast<size_t>(p.QH / p.KH);
     size_t off = 0;
     L.q_code = off; off += sl_align_up(sizeof(uint32_t) * p.B * p.QH * W, 256);
+    L.attn = off;   off += sl_align_up(sl_attn_ws_bytes(p.B, p.QH, p.KH, 1), 256);  // does not depend on k
+    L.n_rows = off; off += sl_align_up(sizeof(int32_t) * p.B, 256);
     L.select = off; off += sl_select_ws_bytes(p.B, p.KH, static_cast<int>(G * p.nbits + 1), p.n_cap);
     L.score = off;  off += sl_align_up(sizeof(int16_t) * p.B * p.KH * static_cast<size_t>(p.n_cap), 256);
     L.lru_fetch = off; off += p.lru_C > 0 ? sl_align_up(sizeof(int32_t) * p.B * p.KH * static_cast<size_t>(p.k), 256) : 0;
-    L.attn = off;   off += sl_attn_ws_bytes(p.B, p.QH, p.KH, p.k);
     L.total = off;
     return L;
 }
@@ -135,6 +139,12 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     const int W = p.nbits / 32, G = p.QH / p.KH;
     uint32_t *q_code = reinterpret_cast<uint32_t *>(ws + L.q_code);
     int16_t *score = reinterpret_cast<int16_t *>(ws + L.score);
+    // Lengths: the hash launch reads seq_lens[b] (the row it appends to) and leaves seq_lens[b] + 1 in
+    // n_rows[b]; scorer, selection and attention read n_rows only, and the attention launch advances
+    // seq_lens at its end.  No launch reads a word that one of its own workgroups writes.  (A subset
+    // of stages without the hash launch works on the row counts the last hash launch left.)
+    int32_t *n_rows = reinterpret_cast<int32_t *>(ws + L.n_rows);
+    const size_t attn_bytes = L.n_rows - L.attn;
 
     // 1. hash q and the new key; append code, K, V
     hash_args ha{};
@@ -159,11 +169,12 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     sl_select_carve(ta, ws + L.select, p.n_cap);
     ha.zero_words = ta.hist;  // the scorer of this step starts from a clean histogram
     ha.zero_count = static_cast<int64_t>(p.B) * p.KH * ta.n_bins * ta.hist_groups;
+    ha.len_out = n_rows;
     // 2. score seq_lens[b] + 1 rows
     hamming_args sa{};
-    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.hist_span = ta.hist_span; sa.seq_lens = p.seq_lens;
+    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.hist_span = ta.hist_span; sa.seq_lens = n_rows;
     sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
-    sa.n_bins = G * p.nbits + 1; sa.len_bias = 1; sa.n = p.n_max; sa.n_cap = p.n_cap;
+    sa.n_bins = G * p.nbits + 1; sa.len_bias = 0; sa.n = p.n_max; sa.n_cap = p.n_cap;
     sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
     if (stages & SL_STAGE_HASH) {
         rc = sl_hash_launch(ha, s);
@@ -175,8 +186,8 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     }
 
     // 3. select
-    ta.score = score; ta.idx = p.idx; ta.seq_lens = p.seq_lens;
-    ta.k = p.k; ta.len_bias = 1; ta.n = p.n_max;
+    ta.score = score; ta.idx = p.idx; ta.seq_lens = n_rows;
+    ta.k = p.k; ta.len_bias = 0; ta.n = p.n_max;
     ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
     // 3. select -- or 3+5 in one launch when there is no LRU in between and the shapes allow
     attn_args aa{};
@@ -194,7 +205,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     const int64_t tail_blocks = (p.n_max + 4095) / 4096;
     const bool fuse_tail = g_fuse_select_attend == 2 || (g_fuse_select_attend == 1 && p.k <= 128 * tail_blocks);
     if (both && p.lru_C == 0 && fuse_tail && sl_select_attend_supported(ta, aa))
-        return sl_select_attend_launch(ta, aa, ws + L.attn, L.total - L.attn, s);
+        return sl_select_attend_launch(ta, aa, ws + L.attn, attn_bytes, s);
     if (stages & SL_STAGE_SELECT) {
         rc = sl_select_launch(ta, s);
         if (rc != SL_OK) return rc;
@@ -230,5 +241,5 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         }
     }
     if (!(stages & SL_STAGE_ATTN)) return SL_OK;
-    return sl_attn_launch(aa, ws + L.attn, L.total - L.attn, s);
+    return sl_attn_launch(aa, ws + L.attn, attn_bytes, s);
 }

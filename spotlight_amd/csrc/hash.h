@@ -24,6 +24,10 @@ struct hash_args {
     int dtype, n_layers, B, d_in, d_hid, nbits, residue;
     uint32_t *zero_words;  // optional: words the launch also clears (next step's histogram)
     int64_t zero_count;
+    // optional [B]: receives code_row[b] + 1 of the last side, i.e. the number of cached rows once this
+    // launch's row is appended.  Later launches of the step read lengths from here, so that no launch
+    // reads a length another workgroup of the same launch advances.
+    int32_t *len_out;
 };
 
 int sl_hash_launch(hash_args a, hipStream_t s);

@@ -165,6 +165,9 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
 
     const float xrow[4] = {x0, x1, x2, x3};
     const int32_t drow[4] = {row0, row1, row2, row3};
+    // the step's row count per batch entry, for the launches that follow (head 0 of the last side)
+    if (a.len_out && sd.code_row && side_i == a.n_sides - 1 && h == 0 && tid < nb)
+        a.len_out[b_lo + tid] = (tid == 0 ? row0 : tid == 1 ? row1 : tid == 2 ? row2 : row3) + 1;
     if (tid < HK_DIN) {
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) xs[rr][tid] = xrow[rr];

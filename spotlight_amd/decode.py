@@ -190,6 +190,24 @@ class LayerDecodeState:
         self.seq_lens.fill_(n0)
         self.host_len = n0
 
+    def load_rows(self, keys: torch.Tensor, vals: torch.Tensor, start: int,
+                  codes: Optional[torch.Tensor] = None) -> None:
+        """Prefill in slabs: rows [start, start + t) of every sequence; lengths are set
+        afterwards with ``set_length``.  Bounds the transient memory of hashing."""
+        t = keys.shape[1]
+        assert start + t < self.n_cap
+        if codes is None:
+            codes = self.hash_k.hash_rows(keys)
+        K.cache_append(self.keys, keys.contiguous(), start=start)
+        K.cache_append(self.vals, vals.contiguous(), start=start)
+        K.cache_append(self.codes, codes.contiguous(), start=start)
+
+    def set_length(self, n: int) -> None:
+        assert 0 <= n < self.n_cap
+        self.seq_lens.fill_(n)
+        self.host_len = n
+        self._graph = None
+
     # -- decode ------------------------------------------------------------------
     def _launch(self, n_max: int, stages: int = _lib.STAGE_ALL) -> None:
         if n_max > self.n_cap:

@@ -361,3 +361,39 @@ def test_decode_step_random_shapes(env, B, QH, KH, n0, k, dtype, kind):
         v_new = torch.randn(B, KH, 128, generator=g).to(dtype)
         out = st.step(q.to(DEV), k_new.to(DEV), v_new.to(DEV))
         _check_step(kernel, st, q, k_new, v_new, out, n0 + step, dtype)
+
+
+def test_budget_changes_on_a_live_lru_state(env):
+    """k lowered and raised between steps on one workspace, with the LRU table on and more than
+    one attention run per (b, kv head): the arrival tickets must stay where they are (and zero)
+    whatever k is, so every step still matches the oracle and the state without a table."""
+    decode, kernel = env
+    dtype = torch.bfloat16
+    B, QH, KH, n0, k_max = 2, 32, 8, 900, 100
+    plain = _make_state(decode, _gen(70), B, QH, KH, n0, 1024, k_max, dtype)
+    lru = _make_state(decode, _gen(70), B, QH, KH, n0, 1024, k_max, dtype, lru=128)
+    g = _gen(71)
+    n = n0
+    for step, k in enumerate([100, 37, 100, 64, 12, 100, 99]):
+        plain.set_k(k)
+        lru.set_k(k)
+        q = torch.randn(B, QH, 128, generator=g).to(dtype)
+        kn = torch.randn(B, KH, 128, generator=g).to(dtype)
+        vn = torch.randn(B, KH, 128, generator=g).to(dtype)
+        a = plain.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).clone()
+        b = lru.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).clone()
+        n += 1
+        hq = lru.hash_q
+        q_code = kernel.hash_mlp_pack(q.to(DEV), hq.w1, hq.b1, hq.w2, hq.b2, hq.residue).cpu().numpy()[:, None]
+        score = orc.hamming_score_u32(q_code, lru.codes[:, :n].cpu().numpy(), "blocked")
+        want_idx = orc.topk_stable(score, k)
+        np.testing.assert_array_equal(lru.selected().cpu().numpy(), want_idx)
+        np.testing.assert_array_equal(plain.selected().cpu().numpy(), want_idx)
+        want = orc.sparse_attention(q.float().numpy(), lru.keys[:, :n].float().cpu().numpy(),
+                                    lru.vals[:, :n].float().cpu().numpy(), want_idx)
+        assert np.abs(b.float().cpu().numpy() - want).max() <= TOL[dtype], (step, k)
+        assert np.abs(a.float().cpu().numpy() - want).max() <= TOL[dtype], (step, k)
+        # every kept row is resident where the table says
+        slot = torch.gather(lru.token_slot, 2, lru.selected().long()).long()
+        assert int(slot.min()) >= 0
+        assert torch.equal(torch.gather(lru.slot_token, 2, slot), lru.selected())

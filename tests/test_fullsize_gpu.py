@@ -46,68 +46,113 @@ def _scores(q_codes, k_codes, KH, G):
     return out
 
 
-@pytest.mark.parametrize("name", list(SHAPES))
-@torch.no_grad()
-def test_full_size_step_properties(decode, name):
-    from spotlight_amd import kernel
-    B, QH, KH, n0, k, dtype, kind, lru = SHAPES[name]
-    G = QH // KH
-    g = torch.Generator(device=DEV).manual_seed(7)
-    cg = torch.Generator().manual_seed(7)
+def _weights(decode, kind, QH, KH, dtype, cg):
     if kind == "mlp":
         hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, DEV, cg, scale=0.05)
         hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, DEV, cg, scale=0.05)
     else:
         hq = decode.HashWeights.random_linear(QH, 128, 128, dtype, DEV, cg)
         hk = hq
-    n_cap = n0 + 64
-    st = decode.LayerDecodeState(B, QH, KH, 128, n_cap, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru)
-    keys = torch.randn((B, n0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
-    vals = torch.randn((B, n0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
-    st.prefill(keys, vals)
-    del keys, vals
+    return hq, hk
+
+
+def check_step_properties(st, q, kn, vn, out, n):
+    """What one decode step must have left behind, whatever the implementation: `st` after the
+    step that appended (kn, vn) as row n - 1 and attended for q; `out` that step's output."""
+    from spotlight_amd import kernel
+    B, QH, KH, k, dtype, lru = st.B, st.QH, st.KH, st.current_k, st.dtype, st.lru_slots
+    hq, hk = st.hash_q, st.hash_k
+    G = QH // KH
+    assert st.seq_lens.tolist() == [n] * B
+    # the appended row is in the cache, with the code of the key hash
+    assert torch.equal(st.keys[:, n - 1], kn) and torch.equal(st.vals[:, n - 1], vn)
+    k_code = kernel.hash_mlp_pack(kn, hk.w1, hk.b1, hk.w2, hk.b2, hk.residue)
+    codes = st.codes[:, :n].view(torch.int32)
+    assert torch.equal(codes[:, n - 1], k_code.view(torch.int32))
+    # selection: k distinct tokens, ascending; nothing left out scores higher than anything
+    # kept; inside the threshold score the kept tokens are the lowest-numbered ones
+    idx = st.selected().long()                                            # [B,KH,k]
+    assert idx.shape == (B, KH, k) and int(idx.min()) >= 0 and int(idx.max()) < n
+    assert bool((idx[..., 1:] > idx[..., :-1]).all())
+    q_code = kernel.hash_mlp_pack(q, hq.w1, hq.b1, hq.w2, hq.b2, hq.residue).view(torch.int32)
+    score = _scores(q_code, codes, KH, G)                                 # [B,KH,n]
+    kept = torch.zeros((B, KH, n), dtype=torch.bool, device=DEV)
+    kept.scatter_(-1, idx, True)
+    thr = torch.where(kept, score, torch.full_like(score, 10 ** 6)).amin(-1, keepdim=True)
+    assert bool((torch.where(kept, torch.full_like(score, -1), score).amax(-1, keepdim=True) <= thr).all())
+    at_thr = score == thr
+    pos = torch.arange(n, device=DEV).expand(B, KH, n)
+    last_kept = torch.where(at_thr & kept, pos, torch.full_like(pos, -1)).amax(-1, keepdim=True)
+    first_left = torch.where(at_thr & ~kept, pos, torch.full_like(pos, n)).amin(-1, keepdim=True)
+    assert bool((last_kept < first_left).all())
+    # the output is softmax attention over exactly those rows
+    bi = torch.arange(B, device=DEV)[:, None, None]
+    hi = torch.arange(KH, device=DEV)[None, :, None]
+    ks = st.keys[bi, idx, hi].float()                                     # [B,KH,k,d]
+    vs = st.vals[bi, idx, hi].float()
+    qg = q.float().reshape(B, KH, G, 128)
+    w = torch.softmax(torch.einsum("bhgd,bhkd->bhgk", qg, ks) / math.sqrt(128.0), dim=-1)
+    want = torch.einsum("bhgk,bhkd->bhgd", w, vs).reshape(B, QH, 128)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert float((out.float() - want).abs().max()) <= tol
+    if lru:
+        # every kept token and the new one are resident, in the slot the map names
+        slot = torch.gather(st.token_slot, 2, idx).long()                 # [B,KH,k]
+        assert int(slot.min()) >= 0
+        assert torch.equal(torch.gather(st.slot_token, 2, slot).long(), idx)
+        assert torch.equal(st.k_res[bi, hi, slot].float(), ks)
+        assert int(st.token_slot[:, :, n - 1].min()) >= 0
+
+
+def _prefilled(decode, B, QH, KH, n0, k, dtype, kind, lru, g, cg, n_cap=None):
+    hq, hk = _weights(decode, kind, QH, KH, dtype, cg)
+    st = decode.LayerDecodeState(B, QH, KH, 128, n_cap or (n0 + 64 + 7) // 8 * 8, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru)
+    slab = max(1, (1 << 21) // (B * KH))   # bounds the transient memory of hashing the rows
+    for s0 in range(0, n0, slab):
+        s1 = min(n0, s0 + slab)
+        keys = torch.randn((B, s1 - s0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+        vals = torch.randn((B, s1 - s0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+        st.load_rows(keys, vals, start=s0)
+    st.set_length(n0)
+    return st
+
+
+def _fresh(g, B, QH, KH, dtype):
+    return tuple(torch.randn((B, h, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype) for h in (QH, KH, KH))
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+@torch.no_grad()
+def test_full_size_step_properties(decode, name):
+    B, QH, KH, n0, k, dtype, kind, lru = SHAPES[name]
+    g = torch.Generator(device=DEV).manual_seed(7)
+    st = _prefilled(decode, B, QH, KH, n0, k, dtype, kind, lru, g, torch.Generator().manual_seed(7))
     for step in range(2):
-        q = torch.randn((B, QH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
-        kn = torch.randn((B, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
-        vn = torch.randn((B, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+        q, kn, vn = _fresh(g, B, QH, KH, dtype)
         out = st.step(q, kn, vn).clone()
-        n = n0 + step + 1
-        assert st.seq_lens.tolist() == [n] * B
-        # the appended row is in the cache, with the code of the key hash
-        assert torch.equal(st.keys[:, n - 1], kn) and torch.equal(st.vals[:, n - 1], vn)
-        k_code = kernel.hash_mlp_pack(kn, hk.w1, hk.b1, hk.w2, hk.b2, hk.residue)
-        codes = st.codes[:, :n].view(torch.int32)
-        assert torch.equal(codes[:, n - 1], k_code.view(torch.int32))
-        # selection: k distinct tokens, ascending; nothing left out scores higher than anything
-        # kept; inside the threshold score the kept tokens are the lowest-numbered ones
-        idx = st.selected().long()                                            # [B,KH,k]
-        assert idx.shape == (B, KH, k) and int(idx.min()) >= 0 and int(idx.max()) < n
-        assert bool((idx[..., 1:] > idx[..., :-1]).all())
-        q_code = kernel.hash_mlp_pack(q, hq.w1, hq.b1, hq.w2, hq.b2, hq.residue).view(torch.int32)
-        score = _scores(q_code, codes, KH, G)                                 # [B,KH,n]
-        kept = torch.zeros((B, KH, n), dtype=torch.bool, device=DEV)
-        kept.scatter_(-1, idx, True)
-        thr = torch.where(kept, score, torch.full_like(score, 10 ** 6)).amin(-1, keepdim=True)
-        assert bool((torch.where(kept, torch.full_like(score, -1), score).amax(-1, keepdim=True) <= thr).all())
-        at_thr = score == thr
-        pos = torch.arange(n, device=DEV).expand(B, KH, n)
-        last_kept = torch.where(at_thr & kept, pos, torch.full_like(pos, -1)).amax(-1, keepdim=True)
-        first_left = torch.where(at_thr & ~kept, pos, torch.full_like(pos, n)).amin(-1, keepdim=True)
-        assert bool((last_kept < first_left).all())
-        # the output is softmax attention over exactly those rows
-        bi = torch.arange(B, device=DEV)[:, None, None]
-        hi = torch.arange(KH, device=DEV)[None, :, None]
-        ks = st.keys[bi, idx, hi].float()                                     # [B,KH,k,d]
-        vs = st.vals[bi, idx, hi].float()
-        qg = q.float().reshape(B, KH, G, 128)
-        w = torch.softmax(torch.einsum("bhgd,bhkd->bhgk", qg, ks) / math.sqrt(128.0), dim=-1)
-        want = torch.einsum("bhgk,bhkd->bhgd", w, vs).reshape(B, QH, 128)
-        tol = 1e-5 if dtype == torch.float32 else 2e-2
-        assert float((out.float() - want).abs().max()) <= tol
-        if lru:
-            # every kept token and the new one are resident, in the slot the map names
-            slot = torch.gather(st.token_slot, 2, idx).long()                 # [B,KH,k]
-            assert int(slot.min()) >= 0
-            assert torch.equal(torch.gather(st.slot_token, 2, slot).long(), idx)
-            assert torch.equal(st.k_res[bi, hi, slot].float(), ks)
-            assert int(st.token_slot[:, :, n - 1].min()) >= 0
+        check_step_properties(st, q, kn, vn, out, n0 + step + 1)
+
+
+@torch.no_grad()
+def test_fused_tail_large_batch_across_block_boundary(decode):
+    """Headline shape at batch 32, one row short of a 4096-row block: the second step opens a
+    ninth block.  The select + attend launch is 2304 workgroups, far more than the device
+    holds at once, so late workgroups start after early ones have finished; every (b, kv head)
+    must still agree on the row count of the step.  Eager steps and graph replays."""
+    B, QH, KH, k, dtype = 32, 32, 8, 655, torch.bfloat16
+    n0 = 8 * 4096 - 1
+    g = torch.Generator(device=DEV).manual_seed(11)
+    st = _prefilled(decode, B, QH, KH, n0, k, dtype, "mlp", 0, g, torch.Generator().manual_seed(11))
+    n = n0
+    for step in range(2):
+        q, kn, vn = _fresh(g, B, QH, KH, dtype)
+        out = st.step(q, kn, vn).clone()
+        n += 1
+        check_step_properties(st, q, kn, vn, out, n)
+    st.capture(8)
+    for step in range(3):
+        q, kn, vn = _fresh(g, B, QH, KH, dtype)
+        st.q_in.copy_(q); st.k_in.copy_(kn); st.v_in.copy_(vn)
+        out = st.replay().clone()
+        n += 1
+        check_step_properties(st, q, kn, vn, out, n)
