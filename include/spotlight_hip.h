@@ -30,7 +30,8 @@ typedef enum {
     SL_ERR_UNSUPPORTED = -3, /* shape/dtype outside what the kernels cover   */
     SL_ERR_ALIGN = -4,       /* pointer or stride not aligned as required    */
     SL_ERR_WORKSPACE = -5,   /* workspace missing or too small               */
-    SL_ERR_LAUNCH = -6       /* hipGetLastError() reported a launch failure  */
+    SL_ERR_LAUNCH = -6,      /* hipGetLastError() reported a launch failure  */
+    SL_ERR_TOO_LARGE = -7    /* problem exceeds a built-in scratch buffer    */
 } sl_status;
 
 typedef enum { SL_F32 = 0, SL_BF16 = 1, SL_F16 = 2 } sl_dtype;
@@ -131,6 +132,22 @@ size_t sl_topk_workspace_bytes(int B, int KH, int max_score, int64_t n);
 int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
                    int32_t *idx, int B, int64_t n, int KH, int k, int max_score,
                    const int32_t *seq_lens, void *ws, size_t ws_bytes, void *stream);
+
+/* The same selection for callers that cannot allocate device memory and have no
+ * workspace to hand over (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  NO counterpart in the reference.  The
+ * scratch is a file-scope device array of SL_TOPK_STATIC_BYTES inside the
+ * library (one copy per GPU, held until the process ends); the call allocates
+ * and frees nothing.  Problems whose sl_topk_workspace_bytes() exceeds
+ * SL_TOPK_STATIC_BYTES are rejected with SL_ERR_TOO_LARGE: use sl_topk_select
+ * then.  All calls on one GPU share that GPU's array, so calls that overlap on
+ * one GPU (different streams or threads) race; calls on one stream do not.
+ * The first call on a device looks the array's address up; make that call
+ * outside graph capture. */
+#define SL_TOPK_STATIC_BYTES (8u << 20)
+int sl_topk_select_static(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                          int32_t *idx, int B, int64_t n, int KH, int k, int max_score,
+                          const int32_t *seq_lens, void *stream);
 
 /* ---- gather --------------------------------------------------------------- */
 

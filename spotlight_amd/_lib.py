@@ -54,6 +54,8 @@ SIGNATURES = {
     "sl_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int64]),
     "sl_topk_select": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_int, c_int, c_int,
                                c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sl_topk_select_static": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_int, c_int, c_int,
+                                      c_void_p, c_void_p]),
     "sl_gather_kv": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64, c_void_p]),
     "sl_cache_append": (c_int, [c_void_p, c_void_p, c_int] + [c_int64] * 5 + [c_void_p, c_void_p]),
     "sl_lru_update": (c_int, [c_void_p] * 11 + [c_int] * 6 + [c_int64, c_int64, c_uint32, c_void_p, c_void_p]),

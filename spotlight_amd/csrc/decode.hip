@@ -79,6 +79,7 @@ extern "C" const char *sl_strerror(int status) {
         case SL_ERR_ALIGN: return "pointer or stride is not aligned as required";
         case SL_ERR_WORKSPACE: return "workspace missing or too small";
         case SL_ERR_LAUNCH: return "kernel launch failed";
+        case SL_ERR_TOO_LARGE: return "problem exceeds the library's built-in scratch buffer: use the entry point that takes a workspace";
         default: return "unknown status";
     }
 }

@@ -33,6 +33,8 @@
 
 #include <string.h>
 
+#include <mutex>
+
 namespace {
 
 constexpr int TK_BLOCK = TK_THREADS * TK_RUN;      // tokens per workgroup
@@ -271,16 +273,10 @@ extern "C" size_t sl_topk_workspace_bytes(int B, int KH, int max_score, int64_t 
     return sl_select_ws_bytes(B, KH, max_score + 1, n);
 }
 
-extern "C" int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
-                              int32_t *idx, int B, int64_t n, int KH, int k, int max_score,
-                              const int32_t *seq_lens, void *ws, size_t ws_bytes, void *stream) {
-    SL_REQUIRE(B >= 0 && n >= 0 && KH > 0 && k >= 0 && max_score >= 0, SL_ERR_SHAPE);
-    if (B == 0 || k == 0) return SL_OK;
-    SL_REQUIRE(score && idx, SL_ERR_NULL);
-    SL_REQUIRE(max_score + 1 <= TK_MAX_BINS, SL_ERR_UNSUPPORTED);
-    SL_REQUIRE(n <= 0x7fffffffLL && B <= 65535, SL_ERR_UNSUPPORTED);
-    SL_REQUIRE(ws && ws_bytes >= sl_topk_workspace_bytes(B, KH, max_score, n), SL_ERR_WORKSPACE);
-    SL_REQUIRE(sl_aligned(ws, 16), SL_ERR_ALIGN);
+namespace {
+
+int topk_select_with(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h, int32_t *idx, int B,
+                     int64_t n, int KH, int k, int max_score, const int32_t *seq_lens, void *ws, hipStream_t s) {
     const int n_bins = max_score + 1;
     int heads_per_group = 16384 / n_bins;  // 64 KiB of LDS bins per workgroup
     if (heads_per_group > KH) heads_per_group = KH;
@@ -291,7 +287,6 @@ extern "C" int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t st
     a.B = B; a.KH = KH; a.k = k; a.n_bins = n_bins; a.len_bias = 0; a.n = n;
     a.stride_b = stride_b; a.stride_n = stride_n; a.stride_h = stride_h;
     sl_select_carve(a, ws, n);
-    hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t hist_words = static_cast<int64_t>(B) * KH * n_bins * a.hist_groups;
     zero_words_kernel<<<dim3(static_cast<unsigned>((hist_words + 255) / 256)), dim3(256), 0, s>>>(a.hist, hist_words);
     if (n > 0) {
@@ -301,4 +296,65 @@ extern "C" int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t st
         if (rc != SL_OK) return rc;
     }
     return sl_select_launch(a, s);
+}
+
+int topk_check_args(const int16_t *score, const int32_t *idx, int B, int64_t n, int KH, int k, int max_score) {
+    SL_REQUIRE(B >= 0 && n >= 0 && KH > 0 && k >= 0 && max_score >= 0, SL_ERR_SHAPE);
+    if (B == 0 || k == 0) return SL_OK;
+    SL_REQUIRE(score && idx, SL_ERR_NULL);
+    SL_REQUIRE(max_score + 1 <= TK_MAX_BINS, SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(n <= 0x7fffffffLL && B <= 65535, SL_ERR_UNSUPPORTED);
+    return SL_OK;
+}
+
+// ---- built-in scratch for callers that cannot allocate ----------------------------------------
+// The array lives in the code object: every device the library runs on holds its own copy, at its
+// own address, until the process ends.  Host code never passes the array's name to a kernel (on
+// the host that name is only a handle): it asks the runtime for the device address once per device
+// and uses that pointer from then on.
+constexpr size_t TK_STATIC_BYTES = SL_TOPK_STATIC_BYTES;
+__device__ __align__(256) unsigned char tk_static_scratch[TK_STATIC_BYTES];
+constexpr int TK_MAX_DEVICES = 64;
+void *g_static_ptr[TK_MAX_DEVICES];
+std::mutex g_static_mutex;
+
+int static_scratch(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TK_MAX_DEVICES) { (void)hipGetLastError(); return SL_ERR_LAUNCH; }
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(tk_static_scratch)) != hipSuccess || !p) { (void)hipGetLastError(); return SL_ERR_LAUNCH; }
+        g_static_ptr[dev] = p;
+    }
+    *out = g_static_ptr[dev];
+    return SL_OK;
+}
+
+}  // namespace
+
+extern "C" int sl_topk_select(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                              int32_t *idx, int B, int64_t n, int KH, int k, int max_score,
+                              const int32_t *seq_lens, void *ws, size_t ws_bytes, void *stream) {
+    const int rc = topk_check_args(score, idx, B, n, KH, k, max_score);
+    if (rc != SL_OK || B == 0 || k == 0) return rc;
+    SL_REQUIRE(ws && ws_bytes >= sl_topk_workspace_bytes(B, KH, max_score, n), SL_ERR_WORKSPACE);
+    SL_REQUIRE(sl_aligned(ws, 16), SL_ERR_ALIGN);
+    return topk_select_with(score, stride_b, stride_n, stride_h, idx, B, n, KH, k, max_score, seq_lens, ws,
+                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int sl_topk_select_static(const int16_t *score, int64_t stride_b, int64_t stride_n, int64_t stride_h,
+                                     int32_t *idx, int B, int64_t n, int KH, int k, int max_score,
+                                     const int32_t *seq_lens, void *stream) {
+    int rc = topk_check_args(score, idx, B, n, KH, k, max_score);
+    if (rc != SL_OK || B == 0 || k == 0) return rc;
+    SL_REQUIRE(sl_topk_workspace_bytes(B, KH, max_score, n) <= TK_STATIC_BYTES, SL_ERR_TOO_LARGE);
+    void *scratch = nullptr;
+    rc = static_scratch(&scratch);
+    if (rc != SL_OK) return rc;
+    // nothing in the scratch has to survive from one call to the next: the histogram copies are
+    // cleared by the first kernel below, everything else is written before it is read
+    return topk_select_with(score, stride_b, stride_n, stride_h, idx, B, n, KH, k, max_score, seq_lens, scratch,
+                            static_cast<hipStream_t>(stream));
 }
