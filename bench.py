@@ -13,7 +13,10 @@ pre-generated pool); replays are timed with the inputs resident in HBM.
 Prints ONE JSON line.  ``value`` is microseconds per step (lower is better);
 ``roofline`` prices the dominant kernel against the 8 TB/s HBM peak of MI355X
 on its algorithmic bytes; ``cpu_baseline`` is the CPU oracle's cached-codes
-decode step timed on this host on a bounded sample of the same workload.
+decode step timed on this host on a bounded sample of the same workload, and
+``cpu_baseline_reference_form`` the reference's literal decode branch (every key
+re-hashed per step, dense masked attention) on the same host.  ``latency_floor``
+is what the step's launches cost when their kernels do nothing.
 """
 from __future__ import annotations
 
@@ -76,6 +79,8 @@ def main():
                     help="also run a plain 256 MiB device copy (reference point for HBM byte counters)")
     ap.add_argument("--host-store", action="store_true",
                     help="keep the full K/V store in pinned host memory behind the LRU table (configs with LRU slots)")
+    ap.add_argument("--floor-only", action="store_true",
+                    help="only measure what the step's launches cost by themselves (near-empty kernels on the step's grids)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-breakdown", action="store_true")
     args = ap.parse_args()
@@ -105,8 +110,16 @@ def main():
     dtype = torch.float32 if c["dtype"] == "f32" else torch.bfloat16
     B, QH, KH, n0, k, d = c["B"], c["QH"], c["KH"], c["n0"], c["k"], 128
 
-    tokens = math.ceil(warmup / L) + math.ceil(steps / L) + 4 + 64   # cache growth incl. the breakdown passes
+    # the timed region is whole tokens (one graph replay = one token = L steps): the number of steps asked
+    # for is rounded to whole tokens, at least one, and the warm-up covers every layer at least once
+    tokens_timed = max(1, round(steps / L))
+    tokens_warm = max(1, math.ceil(warmup / L))
+    steps_timed, steps_warm = tokens_timed * L, tokens_warm * L
+    tokens = tokens_warm + tokens_timed + 4 + 64   # cache growth incl. the breakdown passes
     n_cap = (n0 + tokens + 7) // 8 * 8
+    if args.floor_only:
+        print(json.dumps({"config": args.config, "latency_floor": latency_floor(dev, c, L, n0 + tokens, reps=64)}), flush=True)
+        return
 
     cpu_gen = torch.Generator()
     cpu_gen.manual_seed(0)
@@ -162,31 +175,24 @@ def main():
     n_max = n0 + tokens
     token_graph = capture(lambda: token_body(n_max))
 
-    def run_steps(nsteps):
-        full, rem = divmod(nsteps, L)
-        for _ in range(full):
-            token_graph.replay()
-        if rem:  # a partial token: deliver inputs, then the first `rem` layers, eagerly
-            for i in range(3):
-                torch.index_select(pool[i], 0, tok, out=cur[i])
-            tok.add_(1).remainder_(P)
-            for st in layers[:rem]:
-                st._launch(n_max)
-
-    run_steps(warmup)
+    for _ in range(tokens_warm):
+        token_graph.replay()
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
-    run_steps(steps)
+    for _ in range(tokens_timed):
+        token_graph.replay()
     ev1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     gpu_ms = ev0.elapsed_time(ev1)
-    ms_per_step = wall_ms / steps
+    ms_per_step = wall_ms / steps_timed
     us_per_step = ms_per_step * 1e3
-    n_mid = n0 + (math.ceil(warmup / L) + steps / L / 2)
+    n_mid = n0 + tokens_warm + tokens_timed / 2
     ab = algorithmic_bytes(c, n_mid)
+    for st in layers:   # the graph advanced the lengths on the device; keep the host-side bound in step
+        st.host_len = n0 + tokens_warm + tokens_timed
 
     if args.calibration_copy:
         src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
@@ -248,26 +254,34 @@ def main():
                     "algorithmic_bytes_per_launch": kernels[dominant]["algorithmic_bytes"],
                     "us_per_launch": kernels[dominant]["us"]}
 
-    cpu_baseline = None
+    floor = latency_floor(dev, c, L, n_max)
+
+    cpu_baseline = cpu_reference_form = None
     if not args.no_cpu_baseline:
-        cpu_baseline = cpu_leg(layers[0], c, budget_s=20.0)
+        cpu_baseline = cpu_leg(layers[0], c, budget_s=12.0)
+        cpu_reference_form = cpu_leg_reference_form(layers[0], c, budget_s=12.0)
 
     step_gbps = ab["step"] / us_per_step / 1e3
     out = {
         "metric": "sparse-decode us/step/layer (Llama-3-8B GQA, 32k ctx)" if args.config == "c2"
                   else f"sparse-decode us/step/layer ({args.config})",
         "value": round(us_per_step, 3), "unit": "us/step/layer", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "steps_timed": steps_timed, "warmup_timed": steps_warm,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": c["dtype"], "data": "synthetic",
         "config": {"workload": f"{args.config}: {c['desc']}", "batch": B, "q_heads": QH, "kv_heads": KH,
                    "head_dim": d, "context": n0, "k": k, "code_bits": 128, "hash": c["hash"],
                    "lru_slots": c["lru"], "kv_store": "pinned host memory" if args.host_store else "hbm",
-                   "layers_rotated": L, "graph": "one HIP graph per token"},
-        "gpu_event_ms_per_step": round(gpu_ms / steps, 6),
+                   "layers_rotated": L,
+                   "graph": f"one HIP graph per token ({L} steps); {tokens_timed} replays timed after {tokens_warm} warm-up replays"},
+        "gpu_event_ms_per_step": round(gpu_ms / steps_timed, 6),
         "hbm_gbps": round(step_gbps, 1), "hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(ab["step"]),
         "tokens_per_s": round(B / (ms_per_step * 1e-3 * L), 2), "tokens_per_s_layers": L,
         "kernels": kernels, "roofline": roofline, "cpu_baseline": cpu_baseline,
+        "cpu_baseline_reference_form": cpu_reference_form,
+        "latency_floor": floor,
+        "value_over_floor": round(us_per_step / floor["launches_with_one_load_us"], 2) if floor else None,
     }
     print(json.dumps(out), flush=True)
 
@@ -474,6 +488,88 @@ def profiled_traffic(config, stage):
                     except ValueError:
                         return None
     return None
+
+
+def latency_floor(dev, c, L, n_max, reps=8):
+    """What the step's launches cost by themselves on this machine: a HIP graph of L x (as many dependent
+    launches as the step has, with the step's grids) of a kernel that does nothing, and of one whose lanes do a
+    single dependent load.  us per step-equivalent."""
+    import torch
+
+    from spotlight_amd import _lib
+    lib = _lib.load()
+    B, QH, KH = c["B"], c["QH"], c["KH"]
+    hash_rows = 1
+    while hash_rows < 4 and (QH + KH) * ((B + hash_rows - 1) // hash_rows) > 256:
+        hash_rows *= 2
+    blocks4k = (n_max + 4095) // 4096
+    grids = [((QH + KH) * ((B + hash_rows - 1) // hash_rows), 512),
+             (((n_max * KH + 2047) // 2048) * B, 512)]
+    if c["lru"]:
+        grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
+    elif QH // KH in (1, 2, 4) and n_max <= 65536 and c["k"] <= 128 * blocks4k:
+        grids += [(blocks4k * KH * B, 512)]
+    else:
+        grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
+    table = torch.zeros(1024, dtype=torch.int32, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    res = {"launches_per_step": len(grids), "grids": grids}
+    for name, chain in (("empty_launches_us", 0), ("launches_with_one_load_us", 1)):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            s = torch.cuda.current_stream().cuda_stream
+            for _ in range(L):
+                for blocks, threads in grids:
+                    _lib.check(lib.sl_probe_launch(blocks, threads, table.data_ptr(), sink.data_ptr(), chain, s), "sl_probe_launch")
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        res[name] = round(e0.elapsed_time(e1) * 1e3 / (reps * L), 3)
+        del g
+    return res
+
+
+def cpu_leg_reference_form(st, c, budget_s):
+    """The reference's literal decode branch (spotlight_generation.py:149-215) on this host: hash the query
+    AND every cached key with the per-query-head weights (keys repeat_kv'd), +-1 matmul, per-query-head
+    topk, finfo.min mask, dense SDPA -- one sequence at a time, as the reference asserts batch 1."""
+    import torch
+
+    from oracle import spotlight_oracle as orc
+
+    n = int(st.seq_lens.max().item())
+    B, QH, KH = st.B, st.QH, st.KH
+    G = QH // KH
+    hq = st.hash_q
+    bias = lambda b, width: (b.cpu() if b is not None else torch.zeros(QH, width, dtype=hq.w1.dtype))[None, :, None]
+    ws = [(hq.w1.cpu()[None], bias(hq.b1, hq.d_hid))]
+    if hq.w2 is not None:
+        ws.append((hq.w2.cpu()[None], bias(hq.b2, hq.nbits)))
+    keys = [st.keys[b:b + 1, :n].cpu().permute(0, 2, 1, 3).repeat_interleave(G, dim=1) for b in range(min(B, 2))]
+    vals = [st.vals[b:b + 1, :n].cpu().permute(0, 2, 1, 3).repeat_interleave(G, dim=1) for b in range(min(B, 2))]
+    mask_out = 1.0 - c["k"] / n
+    g = torch.Generator()
+    g.manual_seed(2)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 1 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
+        q = torch.randn(1, QH, 1, 128, generator=g).to(st.dtype)
+        b = len(times) % len(keys)
+        t0 = time.perf_counter()
+        orc.decode_step_reference_form(q, keys[b], vals[b], ws, hq.residue, mask_out)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(med * B * 1e6, 1), "unit": "us/step/layer", "cores": torch.get_num_threads(),
+            "kind": "port", "host_cpus": os.cpu_count(),
+            "sample": f"{len(times)} decode steps of one layer and ONE sequence at n={n} (median"
+                      + (f", multiplied by the batch of {B}" if B > 1 else "") + "), torch CPU restatement of the "
+                      "reference's own decode branch: every cached key re-hashed per step, +-1 matmul, torch.topk, "
+                      "masked dense SDPA"}
 
 
 def cpu_leg(st, c, budget_s):

@@ -288,6 +288,13 @@ enum {
 };
 int sl_decode_stages(const sl_decode_params *p, int stages, void *stream);
 
+/* Measurement aid (no counterpart in the reference): enqueues a kernel of
+ * `blocks` x `threads` lanes that does nothing but `chain` dependent 4-byte loads
+ * per lane from `table` (1024 zero words; NULL allowed when chain == 0).  A
+ * graph of such launches with the decode step's grids measures what the
+ * launches themselves cost on a machine, i.e. the floor under the step. */
+int sl_probe_launch(int blocks, int threads, const uint32_t *table, uint32_t *sink, int chain, void *stream);
+
 /* Zero-fills a workspace with a kernel (safe inside a captured HIP graph). */
 int sl_workspace_init(void *ws, size_t ws_bytes, void *stream);
 

@@ -64,6 +64,7 @@ SIGNATURES = {
     "sl_decode_workspace_bytes": (c_size_t, [C.POINTER(DecodeParams)]),
     "sl_decode_step": (c_int, [C.POINTER(DecodeParams), c_void_p]),
     "sl_decode_stages": (c_int, [C.POINTER(DecodeParams), c_int, c_void_p]),
+    "sl_probe_launch": (c_int, [c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "sl_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
 }
 

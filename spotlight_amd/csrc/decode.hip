@@ -30,6 +30,13 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, ui
     if (i < n_tail) tail[i] = 0;
 }
 
+// Measurement aid: a launch that does nothing but `chain` dependent loads per lane.
+__global__ void probe_kernel(const uint32_t *src, uint32_t *dst, int chain) {
+    uint32_t v = blockIdx.x * blockDim.x + threadIdx.x;
+    for (int i = 0; i < chain; ++i) v = src[v & 1023u];
+    if (v == 0xffffffffu) dst[0] = v;  // never true for the zero-filled table the caller passes
+}
+
 int g_fuse_select_attend = 1;  // sl_tune("fuse_select_attend", 0 | 1 | 2): never, by shape, whenever possible
 
 // Only the attention tickets (head of `attn`) have to stay zero between calls.  Nothing in front of
@@ -91,6 +98,13 @@ extern "C" int sl_tune(const char *key, int value) {
     if (!strcmp(key, "fuse_select_attend") && value >= 0 && value <= 2) { g_fuse_select_attend = value; return SL_OK; }
     if (sl_attn_tune(key, value) == SL_OK || sl_select_tune(key, value) == SL_OK) return SL_OK;
     return sl_hash_tune(key, value);
+}
+
+extern "C" int sl_probe_launch(int blocks, int threads, const uint32_t *table, uint32_t *sink, int chain, void *stream) {
+    SL_REQUIRE(blocks > 0 && threads > 0 && threads <= 1024 && chain >= 0, SL_ERR_SHAPE);
+    if (chain > 0) SL_REQUIRE(table && sink, SL_ERR_NULL);
+    probe_kernel<<<dim3(blocks), dim3(threads), 0, static_cast<hipStream_t>(stream)>>>(table, sink, chain);
+    return sl_check_launch();
 }
 
 extern "C" int sl_host_device_pointer(void *host_ptr, void **device_ptr) {
