@@ -244,8 +244,15 @@ typedef struct {
     int64_t n_max;          /* upper bound of seq_lens[b] + 1 for this call     */
     /* per-step inputs */
     const void *q;          /* [B, QH, d]                                       */
-    const void *k_new;      /* [B, KH, d] post-RoPE                             */
+    const void *k_new;      /* [B, KH, d]                                       */
     const void *v_new;      /* [B, KH, d]                                       */
+    /* rotary embedding (check_and_apply_qk_rope, modify_llama.py:54-80), done  */
+    /* ONCE per token, when it is appended: with rope_inv_freq ([d/2] floats,   */
+    /* theta^(-2i/d)) q and k_new arrive un-rotated and the step rotates both   */
+    /* at position seq_lens[b] (rotate_half convention) before hashing; the     */
+    /* rotated key is what the cache stores.  NULL: q and k_new arrive rotated. */
+    const float *rope_inv_freq;
+    void *q_rot;            /* [B, QH, d] scratch: the rotated queries          */
     /* hash weights; n_layers in {1, 2}; *_k may alias *_q when KH == QH        */
     int n_layers, d_hid, residue;
     const void *w1_q, *b1_q, *w2_q, *b2_q;   /* [QH, ...]                       */

@@ -475,6 +475,20 @@ def _rotate_half(x):
     return torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
 
 
+def apply_rope(x, pos, theta=10000.0):
+    """Rotary embedding of x [B,H,d] at absolute positions pos [B], in x's dtype.
+
+    Restates apply_rotary_pos_emb (spotlight/modifiers/modify_llama.py:54-59) with the
+    cos / sin table of transformers' rotary_emb (inv_freq = theta^(-2i/d), angles in
+    fp32, table cast to x's dtype): x * cos + rotate_half(x) * sin."""
+    d = x.shape[-1]
+    inv_freq = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    ang = torch.as_tensor(pos).to(torch.float32)[:, None] * inv_freq[None, :]
+    emb = torch.cat((ang, ang), dim=-1)
+    cos, sin = emb.cos().to(x.dtype)[:, None, :], emb.sin().to(x.dtype)[:, None, :]
+    return x * cos + _rotate_half(x) * sin
+
+
 def reference_self_attn_forward(hidden_states, kv_cache, q_w, k_w, v_w, o_w, num_heads, num_kv_heads, hash_weights,
                                 residue, draft_enable, mask_out, min_remain, rope_theta=10000.0):
     """spotlight_generation.py:109-226 step by step, for B == 1, on CPU.

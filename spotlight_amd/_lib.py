@@ -27,6 +27,7 @@ class DecodeParams(C.Structure):
         ("nbits", c_int), ("k", c_int), ("head_map", c_int),
         ("n_cap", c_int64), ("n_max", c_int64),
         ("q", c_void_p), ("k_new", c_void_p), ("v_new", c_void_p),
+        ("rope_inv_freq", c_void_p), ("q_rot", c_void_p),
         ("n_layers", c_int), ("d_hid", c_int), ("residue", c_int),
         ("w1_q", c_void_p), ("b1_q", c_void_p), ("w2_q", c_void_p), ("b2_q", c_void_p),
         ("w1_k", c_void_p), ("b1_k", c_void_p), ("w2_k", c_void_p), ("b2_k", c_void_p),

@@ -70,6 +70,7 @@ int validate(const sl_decode_params &p) {
     SL_REQUIRE((p.QH / p.KH) * p.nbits + 1 <= TK_MAX_BINS, SL_ERR_UNSUPPORTED);
     SL_REQUIRE(p.q && p.k_new && p.v_new && p.codes && p.keys && p.vals && p.seq_lens && p.out && p.idx, SL_ERR_NULL);
     SL_REQUIRE(p.w1_q && p.w1_k, SL_ERR_NULL);
+    if (p.rope_inv_freq) SL_REQUIRE(p.q_rot && sl_aligned(p.q_rot, 16), SL_ERR_NULL);
     if (p.lru_C > 0)
         SL_REQUIRE(p.slot_token && p.slot_stamp && p.token_slot && p.k_res && p.v_res && p.slots_out && p.step_counter, SL_ERR_NULL);
     return SL_OK;
@@ -176,7 +177,16 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     sk.codes = p.codes; sk.code_row = p.seq_lens; sk.H = p.KH;
     sk.x_stride_b = static_cast<int64_t>(p.KH) * p.d;
     sk.code_stride_b = p.n_cap * p.KH * W; sk.code_stride_h = W; sk.code_stride_n = static_cast<int64_t>(p.KH) * W;
-    sk.copy_src[0] = p.k_new; sk.copy_dst[0] = p.keys;
+    // with rotary embedding the hash launch rotates q and the new key at position seq_lens[b] first:
+    // the rotated query goes to q_rot (the attention reads it from there), the rotated key into its
+    // cache row (instead of the plain copy of k_new)
+    const bool rope = p.rope_inv_freq != nullptr;
+    ha.rope_inv_freq = p.rope_inv_freq; ha.rope_pos = p.seq_lens;
+    if (rope) {
+        sq.rot_dst = p.q_rot; sq.rot_dst_stride_b = static_cast<int64_t>(p.QH) * p.d; sq.rot_dst_stride_n = 0;
+        sk.rot_dst = p.keys; sk.rot_dst_stride_b = p.n_cap * p.KH * p.d; sk.rot_dst_stride_n = static_cast<int64_t>(p.KH) * p.d;
+    }
+    sk.copy_src[0] = rope ? nullptr : p.k_new; sk.copy_dst[0] = p.keys;
     sk.copy_src[1] = p.v_new; sk.copy_dst[1] = p.vals;
     sk.copy_dst_stride_b = p.n_cap * p.KH * p.d; sk.copy_dst_stride_n = static_cast<int64_t>(p.KH) * p.d;
     select_args ta{};
@@ -206,7 +216,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
     // 3. select -- or 3+5 in one launch when there is no LRU in between and the shapes allow
     attn_args aa{};
-    aa.q = p.q; aa.out = p.out; aa.dtype = p.dtype; aa.B = p.B; aa.QH = p.QH; aa.KH = p.KH; aa.k = p.k;
+    aa.q = rope ? p.q_rot : p.q; aa.out = p.out; aa.dtype = p.dtype; aa.B = p.B; aa.QH = p.QH; aa.KH = p.KH; aa.k = p.k;
     aa.rows = 0; aa.scale = 0.f; aa.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
     const bool whole = stages == SL_STAGE_ALL;  // lengths only advance on a complete step
     aa.bump_lens = whole ? p.seq_lens : nullptr; aa.bump_step = whole ? p.step_counter : nullptr;

@@ -16,6 +16,10 @@ struct hash_side {
     const void *copy_src[2];
     void *copy_dst[2];
     int64_t copy_dst_stride_b, copy_dst_stride_n;
+    // with rotary embedding (hash_args::rope_inv_freq): the rotated input (what is hashed) is also
+    // stored, as [H, d_in] rows at rot_dst + b*rot_dst_stride_b + row[b]*rot_dst_stride_n + h*d_in
+    void *rot_dst;
+    int64_t rot_dst_stride_b, rot_dst_stride_n;
 };
 
 struct hash_args {
@@ -28,6 +32,10 @@ struct hash_args {
     // launch's row is appended.  Later launches of the step read lengths from here, so that no launch
     // reads a length another workgroup of the same launch advances.
     int32_t *len_out;
+    // optional rotary embedding of the inputs of every side before they are hashed (rotate_half
+    // convention): inv_freq [d_in / 2] floats, position of batch entry b = rope_pos[b]
+    const float *rope_inv_freq;
+    const int32_t *rope_pos;
 };
 
 int sl_hash_launch(hash_args a, hipStream_t s);

@@ -115,6 +115,15 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     const float x1 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 1 ? 1 : 0)) * sd.x_stride_b]);
     const float x2 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 2 ? 2 : 0)) * sd.x_stride_b]);
     const float x3 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 3 ? 3 : 0)) * sd.x_stride_b]);
+    // rotary embedding: the partner element (i +- d/2), the frequency and the positions, loaded
+    // whether or not they are used (without rope they re-read what is loaded anyway)
+    const bool rope = a.rope_inv_freq != nullptr;
+    const T *xpart = xh + ((tid + HK_DIN / 2) & (HK_DIN - 1));
+    const float y0 = to_f32(xpart[static_cast<int64_t>(b_lo) * sd.x_stride_b]);
+    const float y1 = to_f32(xpart[static_cast<int64_t>(b_lo + (nb > 1 ? 1 : 0)) * sd.x_stride_b]);
+    const float y2 = to_f32(xpart[static_cast<int64_t>(b_lo + (nb > 2 ? 2 : 0)) * sd.x_stride_b]);
+    const float y3 = to_f32(xpart[static_cast<int64_t>(b_lo + (nb > 3 ? 3 : 0)) * sd.x_stride_b]);
+    const float inv_freq = rope ? a.rope_inv_freq[tid & (HK_DIN / 2 - 1)] : 0.f;
     const int cg = tid % S1::LPR, r = tid / S1::LPR;
     float w1r[S1::PASSES][8];
     {
@@ -146,6 +155,11 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     const int32_t row2 = rowp[sd.code_row ? b_lo + (nb > 2 ? 2 : 0) : 0];
     const int32_t row3 = rowp[sd.code_row ? b_lo + (nb > 3 ? 3 : 0) : 0];
     const int32_t cp_row = rowp[sd.code_row ? cp_b : 0];
+    const int32_t *posp = rope ? a.rope_pos : rowp;
+    const int32_t pos0 = posp[rope ? b_lo : 0];
+    const int32_t pos1 = posp[rope ? b_lo + (nb > 1 ? 1 : 0) : 0];
+    const int32_t pos2 = posp[rope ? b_lo + (nb > 2 ? 2 : 0) : 0];
+    const int32_t pos3 = posp[rope ? b_lo + (nb > 3 ? 3 : 0) : 0];
     const T *src0 = sd.copy_src[0] ? static_cast<const T *>(sd.copy_src[0]) : static_cast<const T *>(sd.x);
     const T *src1 = sd.copy_src[1] ? static_cast<const T *>(sd.copy_src[1]) : static_cast<const T *>(sd.x);
     const int64_t cp_off = static_cast<int64_t>(cp_b) * sd.x_stride_b + h * HK_DIN;
@@ -163,8 +177,31 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
         for (int64_t i = n4 * 4 + wg * HK_THREADS + tid; i < a.zero_count; i += n_wg * HK_THREADS) a.zero_words[i] = 0u;
     }
 
-    const float xrow[4] = {x0, x1, x2, x3};
+    float xrow[4] = {x0, x1, x2, x3};
     const int32_t drow[4] = {row0, row1, row2, row3};
+    if (rope) {
+        // out[i] = x[i] * cos + rot[i] * sin, rot = (-x[d/2:], x[:d/2]); cos / sin and every
+        // product are rounded to T where the torch expression of the reference rounds them
+        const float yrow[4] = {y0, y1, y2, y3};
+        const int32_t prow[4] = {pos0, pos1, pos2, pos3};
+        const float sgn = (tid & (HK_DIN / 2)) ? 1.f : -1.f;
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            float sn, cs;
+            sincosf(static_cast<float>(prow[rr]) * inv_freq, &sn, &cs);
+            cs = round_to<T>(cs);
+            sn = round_to<T>(sn);
+            xrow[rr] = round_to<T>(round_to<T>(xrow[rr] * cs) + round_to<T>(sgn * yrow[rr] * sn));
+        }
+        if (sd.rot_dst && tid < HK_DIN) {
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr)
+                if (b_lo + rr < b_hi)
+                    static_cast<T *>(sd.rot_dst)[static_cast<int64_t>(b_lo + rr) * sd.rot_dst_stride_b +
+                                                 static_cast<int64_t>(sd.code_row ? drow[rr] : 0) * sd.rot_dst_stride_n +
+                                                 h * HK_DIN + tid] = from_f32<T>(xrow[rr]);
+        }
+    }
     // the step's row count per batch entry, for the launches that follow (head 0 of the last side)
     if (a.len_out && sd.code_row && side_i == a.n_sides - 1 && h == 0 && tid < nb)
         a.len_out[b_lo + tid] = (tid == 0 ? row0 : tid == 1 ? row1 : tid == 2 ? row2 : row3) + 1;
@@ -328,6 +365,7 @@ int sl_hash_launch(hash_args a, hipStream_t s) {
     if (a.n_layers == 1) SL_REQUIRE(a.nbits == a.d_hid, SL_ERR_SHAPE);
     if (a.residue) SL_REQUIRE(a.d_hid == a.d_in && (a.n_layers == 1 || a.nbits == a.d_hid), SL_ERR_SHAPE);
     SL_REQUIRE(a.B <= 65535, SL_ERR_UNSUPPORTED);
+    if (a.rope_inv_freq) SL_REQUIRE(a.rope_pos && sl_aligned(a.rope_inv_freq, 4), SL_ERR_NULL);
     int Htot = 0;
     for (int i = 0; i < a.n_sides; ++i) {
         const hash_side &sd = a.side[i];

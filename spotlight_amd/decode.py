@@ -93,7 +93,8 @@ class HashWeights:
 class LayerDecodeState:
     def __init__(self, batch_size: int, num_heads: int, num_kv_heads: int, head_dim: int, n_cap: int, k: int,
                  hash_q: HashWeights, hash_k: HashWeights, dtype=torch.bfloat16, device="cuda",
-                 head_map: str = "blocked", lru_slots: int = 0, inputs=None, host_store: bool = False):
+                 head_map: str = "blocked", lru_slots: int = 0, inputs=None, host_store: bool = False,
+                 rope_theta: Optional[float] = None, rope_inv_freq: Optional[torch.Tensor] = None):
         assert head_dim == 128, "the attention kernel covers head_dim 128"
         assert n_cap % 8 == 0, "n_cap must be a multiple of 8"
         assert hash_q.nbits == hash_k.nbits and hash_q.n_layers == hash_k.n_layers
@@ -128,6 +129,16 @@ class LayerDecodeState:
         assert self.q_in.shape == (B, QH, d) and self.k_in.shape == (B, KH, d) and self.v_in.shape == (B, KH, d)
         assert all(t.is_contiguous() and t.dtype == dtype for t in inputs)
         self.out = torch.zeros((B, QH, d), dtype=dtype, device=dev)
+        # rotary embedding inside the step: q and k_new are handed over UN-rotated and the hash launch
+        # rotates them at position seq_lens[b] (the reference re-rotates the whole cache every step,
+        # spotlight_generation.py:139-141; here a key is rotated once, when it is appended)
+        if rope_inv_freq is None and rope_theta is not None:
+            rope_inv_freq = 1.0 / (rope_theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        self.rope_inv_freq = None
+        if rope_inv_freq is not None:
+            self.rope_inv_freq = rope_inv_freq.to(device=dev, dtype=torch.float32).contiguous()
+            assert self.rope_inv_freq.shape == (d // 2,)
+            self.q_rot = torch.zeros((B, QH, d), dtype=dtype, device=dev)
         self.idx = torch.full((B, KH, k), -1, dtype=torch.int32, device=dev)
         self.host_len = 0  # upper bound of seq_lens, tracked on the host for grid sizing
         self.lru_slots = lru_slots
@@ -159,6 +170,8 @@ class LayerDecodeState:
         p.head_map = K._HEAD_MAPS[self.head_map]
         p.n_cap, p.n_max = self.n_cap, 1
         p.q, p.k_new, p.v_new = self.q_in.data_ptr(), self.k_in.data_ptr(), self.v_in.data_ptr()
+        if self.rope_inv_freq is not None:
+            p.rope_inv_freq, p.q_rot = self.rope_inv_freq.data_ptr(), self.q_rot.data_ptr()
         hq, hk = self.hash_q, self.hash_k
         p.n_layers, p.d_hid, p.residue = hq.n_layers, hq.d_hid, int(hq.residue)
         ptr = lambda t: t.data_ptr() if t is not None else None
@@ -250,7 +263,8 @@ class LayerDecodeState:
         return self.idx.view(-1)[: self.B * self.KH * k].view(self.B, self.KH, k)
 
     def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor) -> torch.Tensor:
-        """One decode step: q [B,QH,d], k_new/v_new [B,KH,d] (post-RoPE).
+        """One decode step: q [B,QH,d], k_new/v_new [B,KH,d] (post-RoPE, or un-rotated when the
+        state was built with ``rope_theta`` / ``rope_inv_freq``).
         Returns the attention output [B,QH,d] (a buffer reused by the next step)."""
         with torch.cuda.device(self.device):
             if q is not self.q_in:

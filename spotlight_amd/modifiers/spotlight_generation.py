@@ -12,8 +12,9 @@ What differs is what happens to the cache, which callers treat as opaque
 (``model_model_forward`` only threads it through, :66-75):
 
 * keys are rotated ONCE, when they are appended, and stored post-RoPE with
-  their packed 128-bit code; the reference stores pre-RoPE keys and re-rotates
-  and re-hashes the whole cache every step (:139-141, :14-17);
+  their packed 128-bit code (for a decoded token the HIP step does the rotation
+  itself, inside its hash launch); the reference stores pre-RoPE keys and
+  re-rotates and re-hashes the whole cache every step (:139-141, :14-17);
 * K/V stay at kv-head granularity ``[B, n_cap, KH, d]``; the reference stores
   them ``repeat_kv``-expanded (:128-136);
 * the decode branch (:143-215) runs as the fused HIP step instead of
@@ -144,14 +145,24 @@ class SpotlightKV:
         self.length += t
 
 
-def _dense_attention(q, keys, vals, causal):
-    """q [B,t,QH,d], keys/vals [B,n,KH,d] -> [B,t,QH,d]; torch SDPA with grouped heads."""
+def _dense_attention(q, keys, vals):
+    """q [B,t,QH,d] = the LAST t positions of keys/vals [B,n,KH,d] -> [B,t,QH,d]; torch SDPA
+    with grouped heads.  Row i of the chunk sees the n - t earlier rows and rows 0..i of the
+    chunk (the mask of modify_llama.py:132-143)."""
     B, t, QH, d = q.shape
-    KH = keys.shape[2]
+    n, KH = keys.shape[1], keys.shape[2]
     G = QH // KH
     kk = keys.permute(0, 2, 1, 3).repeat_interleave(G, dim=1)
     vv = vals.permute(0, 2, 1, 3).repeat_interleave(G, dim=1)
-    o = torch.nn.functional.scaled_dot_product_attention(q.permute(0, 2, 1, 3), kk, vv, is_causal=causal)
+    qq = q.permute(0, 2, 1, 3)
+    if t == 1:
+        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv)
+    elif t == n:
+        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, is_causal=True)
+    else:   # a chunk behind a non-empty cache: is_causal would align the triangle top-left
+        col = torch.arange(n, device=q.device)[None, :]
+        row = torch.arange(n - t, n, device=q.device)[:, None]
+        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, attn_mask=col <= row)
     return o.permute(0, 2, 1, 3)
 
 
@@ -173,10 +184,15 @@ def self_attn_forward(self, hidden_states: torch.Tensor, kv_cache=None):
     vals = self.v_proj(hidden_states).unflatten(-1, (KH, d))
 
     start = 0 if kv_cache is None else kv_cache.length
-    pos = torch.arange(start, start + t, device=dev)
-    cos, sin = rope_tables(pos, d, float(getattr(cfg, "rope_theta", 10000.0)), dtype)
-    ques = apply_rope(ques, cos, sin)
-    keys = apply_rope(keys, cos, sin)     # rotated once, here; stored post-RoPE
+    theta = float(getattr(cfg, "rope_theta", 10000.0))
+    # one new token of a sparse layer: the HIP step rotates q and the new key itself (at the
+    # position it reads from the device-side length), so they are handed over un-rotated
+    fused_rope = sparse and t == 1 and kv_cache is not None and kv_cache.length > 0
+    if not fused_rope:
+        pos = torch.arange(start, start + t, device=dev)
+        cos, sin = rope_tables(pos, d, theta, dtype)
+        ques = apply_rope(ques, cos, sin)
+        keys = apply_rope(keys, cos, sin)     # rotated once, here; stored post-RoPE
     if sparse and per_qhead:              # the reference's repeat_kv (:128-129)
         keys = keys.repeat_interleave(G, dim=2)
         vals = vals.repeat_interleave(G, dim=2)
@@ -191,20 +207,22 @@ def self_attn_forward(self, hidden_states: torch.Tensor, kv_cache=None):
             hk = hq if per_qhead or KH == QH else self.hash_fn_k.hash_weights()
             k_cap = num_remain(n_cap, dk["mask_out"], dk["min_remain"])
             state = LayerDecodeState(B, QH, KHc, d, n_cap, k_cap, hq, hk,
-                                     dtype=dtype, device=dev, head_map="blocked")
+                                     dtype=dtype, device=dev, head_map="blocked", rope_theta=theta)
         kv_cache = SpotlightKV(B, QH, KHc, d, n_cap, dtype, dev, state)
 
     if t > 1 or not sparse or kv_cache.length == 0:
         # prefill (the draft is not used there, :145) and dense layers
         if kv_cache.state is not None:
-            if kv_cache.length != 0:
-                raise NotImplementedError("chunked prefill of a sparse layer")
-            kv_cache.state.prefill(keys.contiguous(), vals.contiguous())
-            kv_cache.length = t
+            # rows, values and their codes go behind what is cached (chunked prefill included)
+            if kv_cache.length + t >= kv_cache.n_cap:
+                raise RuntimeError(f"cache capacity {kv_cache.n_cap} exceeded")
+            kv_cache.state.load_rows(keys.contiguous(), vals.contiguous(), start=kv_cache.length)
+            kv_cache.state.set_length(kv_cache.length + t)
+            kv_cache.length += t
         else:
             kv_cache.append_dense(keys, vals)
         n = kv_cache.length
-        out = _dense_attention(ques, kv_cache.keys[:, :n], kv_cache.vals[:, :n], causal=t > 1)
+        out = _dense_attention(ques, kv_cache.keys[:, :n], kv_cache.vals[:, :n])
     else:
         st = kv_cache.state
         n = kv_cache.length + 1
@@ -217,7 +235,7 @@ def self_attn_forward(self, hidden_states: torch.Tensor, kv_cache=None):
             # benchmark mode (spotlight_evaluation.py:303-316): IoU of the selected rows
             # against the true top-k of q.k, per query head, averaged over the batch
             from ..iou import selection_iou
-            self.ratios = selection_iou(st.selected(), ques[:, 0], kv_cache.keys[:, :n], k).mean(dim=0).tolist()
+            self.ratios = selection_iou(st.selected(), st.q_rot, kv_cache.keys[:, :n], k).mean(dim=0).tolist()
 
     attn_output = self.o_proj(out.reshape(B, t, hidden))
     return attn_output, kv_cache

@@ -397,3 +397,54 @@ def test_budget_changes_on_a_live_lru_state(env):
         slot = torch.gather(lru.token_slot, 2, lru.selected().long()).long()
         assert int(slot.min()) >= 0
         assert torch.equal(torch.gather(lru.slot_token, 2, slot), lru.selected())
+
+
+@pytest.mark.parametrize("dtype,lru", [(torch.float32, 0), (torch.bfloat16, 0), (torch.float16, 0), (torch.bfloat16, 64)])
+def test_decode_step_rotates_new_query_and_key(env, dtype, lru):
+    """Rotary embedding inside the step (modify_llama.py:54-80): q and k_new go in un-rotated, the
+    step rotates both at position seq_lens[b], hashes and attends with the rotated vectors and
+    stores the rotated key.  Rotated values against the oracle's apply_rope; everything
+    downstream against the oracle on the values the GPU holds."""
+    decode, kernel = env
+    theta = 5e5
+    B, QH, KH, n0, k = 2, 32, 8, 700, 40
+    g = _gen(123)
+    hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, DEV, g, scale=0.05)
+    hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, DEV, g, scale=0.05)
+    st = decode.LayerDecodeState(B, QH, KH, 128, 1024, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru, rope_theta=theta)
+    st.prefill(torch.randn(B, n0, KH, 128, generator=g).to(dtype).to(DEV), torch.randn(B, n0, KH, 128, generator=g).to(dtype).to(DEV))
+    tol = TOL[dtype]
+    for step in range(3):
+        q = torch.randn(B, QH, 128, generator=g).to(dtype)
+        kn = torch.randn(B, KH, 128, generator=g).to(dtype)
+        vn = torch.randn(B, KH, 128, generator=g).to(dtype)
+        out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV))
+        n = n0 + step + 1
+        pos = [n - 1] * B
+        q_rot, k_row = st.q_rot.cpu(), st.keys[:, n - 1].cpu()
+        assert (q_rot.float() - orc.apply_rope(q, pos, theta).float()).abs().max() <= tol
+        assert (k_row.float() - orc.apply_rope(kn, pos, theta).float()).abs().max() <= tol
+        _check_step(kernel, st, q_rot, k_row, vn, out, n - 1, dtype)
+
+
+def test_rotation_uses_each_sequence_s_own_position(env):
+    decode, kernel = env
+    dtype, theta = torch.bfloat16, 10000.0
+    B, QH, KH = 5, 8, 2
+    g = _gen(124)
+    hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, DEV, g, scale=0.05)
+    hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, DEV, g, scale=0.05)
+    st = decode.LayerDecodeState(B, QH, KH, 128, 40000, 16, hq, hk, dtype=dtype, device=DEV, rope_theta=theta)
+    st.prefill(torch.randn(B, 64, KH, 128, generator=g).to(dtype).to(DEV), torch.randn(B, 64, KH, 128, generator=g).to(dtype).to(DEV))
+    lens = [64, 0, 5, 39990, 8191]
+    st.seq_lens.copy_(torch.tensor(lens, dtype=torch.int32))
+    st.host_len = max(lens)
+    q = torch.randn(B, QH, 128, generator=g).to(dtype)
+    kn = torch.randn(B, KH, 128, generator=g).to(dtype)
+    vn = torch.randn(B, KH, 128, generator=g).to(dtype)
+    st.step(q.to(DEV), kn.to(DEV), vn.to(DEV))
+    assert (st.q_rot.cpu().float() - orc.apply_rope(q, lens, theta).float()).abs().max() <= 2e-2
+    k_rows = torch.stack([st.keys[b, l].cpu() for b, l in enumerate(lens)])
+    assert (k_rows.float() - orc.apply_rope(kn, lens, theta).float()).abs().max() <= 2e-2
+    assert torch.equal(st.q_rot[1].cpu(), q[1])            # position 0: the identity
+    assert st.seq_lens.tolist() == [l + 1 for l in lens]

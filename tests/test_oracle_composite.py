@@ -18,13 +18,18 @@ def _gen(seed):
     return g
 
 
-def _rope_complex(x, pos, theta):
-    """x [H, t, d] float64 numpy, pos [t]: pairs (i, i + d/2) rotated by pos * theta^(-2i/d)."""
+def _rope_complex(x, pos, theta, fp32_angles=False):
+    """x [H, t, d] float64 numpy, pos [t]: pairs (i, i + d/2) rotated by pos * theta^(-2i/d).
+    fp32_angles: the angle is the float32 product of float32 factors, as in transformers' table."""
     H, t, d = x.shape
     half = d // 2
     freq = theta ** (-np.arange(half, dtype=np.float64) * 2.0 / d)
+    ang = np.asarray(pos, dtype=np.float64)[:, None] * freq[None, :]
+    if fp32_angles:
+        f32 = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).numpy()   # the table's definition
+        ang = (np.asarray(pos, dtype=np.float32)[:, None] * f32[None, :]).astype(np.float64)
     z = x[..., :half] + 1j * x[..., half:]
-    z = z * np.exp(1j * np.asarray(pos, dtype=np.float64)[:, None] * freq[None, :])[None]
+    z = z * np.exp(1j * ang)[None]
     return np.concatenate([z.real, z.imag], axis=-1)
 
 
@@ -195,3 +200,14 @@ def test_reference_form_budget_and_mask_are_the_reference_s():
         sel = idx[0, h, 0]
         p = torch.softmax(K[0, h, sel].double() @ q[0, h, 0].double() / math.sqrt(d), dim=0)
         np.testing.assert_allclose(out[0, h, 0].numpy(), (p @ V[0, h, sel].double()).numpy(), atol=1e-5)
+
+
+def test_apply_rope_is_the_complex_rotation():
+    g = _gen(3)
+    x = torch.randn(3, 5, 64, generator=g)
+    pos = [0, 7, 31999]
+    got = orc.apply_rope(x, pos, theta=5e5).double().numpy()
+    for b, p in enumerate(pos):
+        want = _rope_complex(x[b].double().numpy()[:, None, :], [p], 5e5, fp32_angles=True)[:, 0]
+        np.testing.assert_allclose(got[b], want, atol=2e-5)
+    assert torch.equal(orc.apply_rope(x, [0, 0, 0]), x)
