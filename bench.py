@@ -286,136 +286,172 @@ def main():
     print(json.dumps(out), flush=True)
 
 
-def run_e2e(args):
-    """c5: a random-init Llama-3-8B (32 layers, hidden 4096, 32 q / 8 kv heads, MLP 14336,
-    vocab 128256, rope theta 5e5), batch 4, 32768-token prompt prefilled densely, then
-    greedy decoding with layers 0-1 dense and layers 2.. on the sparse step (k = 655,
-    MLP hash 128-256-128 per query head and per kv head).  One decoded token for the
-    whole batch and all layers is ONE captured HIP graph (positions and lengths live on
-    the device); `value` is decoded tokens per second over the timed replays."""
-    import torch
-    import torch.nn.functional as F
+class E2EModel:
+    """Random-init Llama-shaped decoder (RMSNorm, rotary GQA attention, SiLU-gated MLP; defaults are
+    Llama-3-8B's dims: hidden 4096, 32 q / 8 kv heads of 128, MLP 14336, vocab 128256, rope theta 5e5)
+    whose layers in ``fix_layers`` attend densely and whose other layers run the sparse HIP step
+    (k rows kept, MLP hash 128-256-128 per query head and per kv head).  It stands for the loop of
+    the reference's ``generate`` (spotlight_generation.py:470-495) with dense layers 0-1
+    (config/llama3-8b-spotlight-generation.json).  ``step_body`` is one decoded token for the
+    whole batch and is capturable as one HIP graph: positions and lengths live on the device, and
+    the sparse step rotates q and the new key itself."""
 
-    from spotlight_amd import decode, kernel
+    def __init__(self, L=32, B=4, n0=32768, n_cap=None, k=655, fix_layers=(0, 1), hidden=4096, inter=14336,
+                 vocab=128256, QH=32, KH=8, theta=5e5, seed=0):
+        import torch
 
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    dt = torch.bfloat16
-    B, n0, QH, KH, d, hidden, inter, vocab, theta, k = 4, 32768, 32, 8, 128, 4096, 14336, 128256, 5e5, 655
-    L = args.layers or 32
-    steps = args.steps if args.steps is not None else 512
-    warmup = args.warmup if args.warmup is not None else 8
-    fix_layers = (0, 1)
-    n_cap = (n0 + steps + warmup + 16 + 7) // 8 * 8
-    g = torch.Generator(device=dev)
-    g.manual_seed(0)
-    cg = torch.Generator()
-    cg.manual_seed(0)
-    rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * 0.02).to(dt)
-    embed, lm_head = rnd(vocab, hidden), rnd(vocab, hidden)
-    layers = []
-    for li in range(L):
-        w = dict(wq=rnd(QH * d, hidden), wk=rnd(KH * d, hidden), wv=rnd(KH * d, hidden), wo=rnd(hidden, QH * d),
-                 wg=rnd(inter, hidden), wu=rnd(inter, hidden), wd=rnd(hidden, inter),
-                 n1=torch.ones(hidden, device=dev, dtype=dt), n2=torch.ones(hidden, device=dev, dtype=dt))
-        if li in fix_layers:
-            w["kc"] = torch.zeros((B, KH, n_cap, d), device=dev, dtype=dt)   # head-major: SDPA reads it in place
-            w["vc"] = torch.zeros((B, KH, n_cap, d), device=dev, dtype=dt)
-        else:
-            hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dt, dev, cg)
-            hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dt, dev, cg)
-            w["st"] = decode.LayerDecodeState(B, QH, KH, d, n_cap, k, hq, hk, dtype=dt, device=dev)
-        layers.append(w)
-    norm_f = torch.ones(hidden, device=dev, dtype=dt)
-    inv_freq = 1.0 / (theta ** (torch.arange(0, d, 2, device=dev, dtype=torch.float32) / d))
+        from spotlight_amd import decode
+        self.dev = dev = torch.device("cuda:0")
+        self.dt = dt = torch.bfloat16
+        self.L, self.B, self.n0, self.k, self.QH, self.KH, self.d = L, B, n0, k, QH, KH, 128
+        self.hidden, self.vocab, self.theta = hidden, vocab, theta
+        self.n_cap = n_cap or (n0 + 1024 + 7) // 8 * 8
+        d = self.d
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        cg = torch.Generator()
+        cg.manual_seed(seed)
+        self.g = g
+        rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * 0.02).to(dt)
+        self.embed, self.lm_head = rnd(vocab, hidden), rnd(vocab, hidden)
+        self.layers = []
+        for li in range(L):
+            w = dict(wq=rnd(QH * d, hidden), wk=rnd(KH * d, hidden), wv=rnd(KH * d, hidden), wo=rnd(hidden, QH * d),
+                     wg=rnd(inter, hidden), wu=rnd(inter, hidden), wd=rnd(hidden, inter),
+                     n1=torch.ones(hidden, device=dev, dtype=dt), n2=torch.ones(hidden, device=dev, dtype=dt))
+            if li in fix_layers:
+                w["kc"] = torch.zeros((B, KH, self.n_cap, d), device=dev, dtype=dt)   # head-major: read in place
+                w["vc"] = torch.zeros((B, KH, self.n_cap, d), device=dev, dtype=dt)
+            else:
+                hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dt, dev, cg)
+                hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dt, dev, cg)
+                w["st"] = decode.LayerDecodeState(B, QH, KH, d, self.n_cap, k, hq, hk, dtype=dt, device=dev,
+                                                  rope_theta=theta)
+            self.layers.append(w)
+        self.norm_f = torch.ones(hidden, device=dev, dtype=dt)
+        self.inv_freq = 1.0 / (theta ** (torch.arange(0, d, 2, device=dev, dtype=torch.float32) / d))
+        self.tok = torch.zeros((B,), dtype=torch.int64, device=dev)
+        self.logits = torch.zeros((B, vocab), dtype=torch.float32, device=dev)   # of the last decoded token
+        self.pos = torch.full((1,), n0, dtype=torch.int64, device=dev)
+        self.col = torch.arange(self.n_cap, device=dev)
+        self.sparse = [w["st"] for w in self.layers if "st" in w]
 
-    def rms(x, w):
+    def rms(self, x, w):
+        import torch
         xf = x.float()
-        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).to(dt) * w
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).to(self.dt) * w
 
-    def rope(x, pos):   # x [..., t, H, d], pos [t] (device)
-        ang = pos.float()[:, None] * inv_freq[None, :]
+    def rope(self, x, pos):   # x [..., t, H, d], pos [t] (device)
+        import torch
+        d = self.d
+        ang = pos.float()[:, None] * self.inv_freq[None, :]
         emb = torch.cat((ang, ang), dim=-1)
-        cos, sin = emb.cos().to(dt)[:, None, :], emb.sin().to(dt)[:, None, :]
+        cos, sin = emb.cos().to(self.dt)[:, None, :], emb.sin().to(self.dt)[:, None, :]
         rot = torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
         return x * cos + rot * sin
 
-    def mlp(w, h):
+    def mlp(self, w, h):
+        import torch.nn.functional as F
         return (F.silu(h @ w["wg"].T) * (h @ w["wu"].T)) @ w["wd"].T
 
-    # ---- prefill: dense causal attention in every layer (the draft is not used there), one sequence at a time
-    t_pre = time.perf_counter()
-    pos0 = torch.arange(n0, device=dev)
-    first = torch.empty((B,), dtype=torch.int64, device=dev)
-    with torch.no_grad():
-        for b in range(B):
-            ids = torch.randint(0, vocab, (n0,), generator=g, device=dev)
-            x = embed[ids]                                                   # [n0, hidden]
-            for w in layers:
-                h = rms(x, w["n1"])
-                q = rope((h @ w["wq"].T).view(n0, QH, d), pos0)
-                kk = rope((h @ w["wk"].T).view(n0, KH, d), pos0)
-                vv = (h @ w["wv"].T).view(n0, KH, d)
-                o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], kk.transpose(0, 1)[None],
-                                                   vv.transpose(0, 1)[None], is_causal=True, enable_gqa=True)
-                x = x + o[0].transpose(0, 1).reshape(n0, QH * d) @ w["wo"].T
-                x = x + mlp(w, rms(x, w["n2"]))
-                if "st" in w:
-                    st = w["st"]
-                    st.keys[b, :n0] = kk
-                    st.vals[b, :n0] = vv
-                    kernel.cache_append(st.codes[b:b + 1], st.hash_k.hash_rows(kk[None]), start=0)
-                else:
-                    w["kc"][b, :, :n0] = kk.transpose(0, 1)
-                    w["vc"][b, :, :n0] = vv.transpose(0, 1)
-            first[b] = (rms(x[-1:], norm_f) @ lm_head.T).float().argmax(dim=-1)[0]
-            del x, h, q, kk, vv, o
-        for w in layers:
-            if "st" in w:
-                w["st"].seq_lens.fill_(n0)
-                w["st"].host_len = n0
-    torch.cuda.synchronize()
-    prefill_s = time.perf_counter() - t_pre
+    def prefill(self):
+        """Dense causal attention in every layer (the draft is not used there), one sequence at a
+        time; sparse layers also get the codes of their keys.  Returns the seconds it took."""
+        import torch
+        import torch.nn.functional as F
 
-    # ---- one decoded token = one graph
-    tok = first.clone()
-    pos = torch.full((1,), n0, dtype=torch.int64, device=dev)
-    n_max = n_cap
-    col = torch.arange(n_cap, device=dev)
+        from spotlight_amd import kernel
+        B, n0, QH, KH, d, dev = self.B, self.n0, self.QH, self.KH, self.d, self.dev
+        t_pre = time.perf_counter()
+        pos0 = torch.arange(n0, device=dev)
+        with torch.no_grad():
+            for b in range(B):
+                ids = torch.randint(0, self.vocab, (n0,), generator=self.g, device=dev)
+                x = self.embed[ids]                                                   # [n0, hidden]
+                for w in self.layers:
+                    h = self.rms(x, w["n1"])
+                    q = self.rope((h @ w["wq"].T).view(n0, QH, d), pos0)
+                    kk = self.rope((h @ w["wk"].T).view(n0, KH, d), pos0)
+                    vv = (h @ w["wv"].T).view(n0, KH, d)
+                    o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], kk.transpose(0, 1)[None],
+                                                       vv.transpose(0, 1)[None], is_causal=True, enable_gqa=True)
+                    x = x + o[0].transpose(0, 1).reshape(n0, QH * d) @ w["wo"].T
+                    x = x + self.mlp(w, self.rms(x, w["n2"]))
+                    if "st" in w:
+                        st = w["st"]
+                        st.keys[b, :n0] = kk
+                        st.vals[b, :n0] = vv
+                        kernel.cache_append(st.codes[b:b + 1], st.hash_k.hash_rows(kk[None]), start=0)
+                    else:
+                        w["kc"][b, :, :n0] = kk.transpose(0, 1)
+                        w["vc"][b, :, :n0] = vv.transpose(0, 1)
+                self.tok[b] = (self.rms(x[-1:], self.norm_f) @ self.lm_head.T).float().argmax(dim=-1)[0]
+                del x, h, q, kk, vv, o
+            for st in self.sparse:
+                st.set_length(n0)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t_pre
 
-    def step_body():
-        x = embed[tok]                                                       # [B, hidden]
-        for w in layers:
-            h = rms(x, w["n1"])
-            q = rope((h @ w["wq"].T).view(B, 1, QH, d), pos)[:, 0]
-            kk = rope((h @ w["wk"].T).view(B, 1, KH, d), pos)[:, 0]
+    def step_body(self):
+        import torch
+        B, QH, KH, d, dt = self.B, self.QH, self.KH, self.d, self.dt
+        x = self.embed[self.tok]                                                       # [B, hidden]
+        for w in self.layers:
+            h = self.rms(x, w["n1"])
+            q = (h @ w["wq"].T).view(B, QH, d)
+            kk = (h @ w["wk"].T).view(B, KH, d)
             vv = (h @ w["wv"].T).view(B, KH, d)
             if "st" in w:
-                st = w["st"]
+                st = w["st"]          # un-rotated q and k: the step rotates them at its own position
                 st.q_in.copy_(q)
                 st.k_in.copy_(kk)
                 st.v_in.copy_(vv)
-                st._launch(n_max)
+                st._launch(self.n_cap)
                 o = st.out.reshape(B, QH * d)
             else:
-                w["kc"].index_copy_(2, pos, kk[:, :, None])
-                w["vc"].index_copy_(2, pos, vv[:, :, None])
+                q = self.rope(q[:, None], self.pos)[:, 0]
+                kk = self.rope(kk[:, None], self.pos)[:, 0]
+                w["kc"].index_copy_(2, self.pos, kk[:, :, None])
+                w["vc"].index_copy_(2, self.pos, vv[:, :, None])
                 # dense decode attention as two batched GEMMs per kv head group (the G query heads of
                 # a kv head are the G rows of the left operand: no K/V expansion, K and V read once)
                 sc = torch.matmul(q.view(B, KH, QH // KH, d), w["kc"].transpose(2, 3)).float() * (d ** -0.5)
-                sc = sc.masked_fill((col > pos)[None, None, None, :], float("-inf"))
+                sc = sc.masked_fill((self.col > self.pos)[None, None, None, :], float("-inf"))
                 o = torch.matmul(torch.softmax(sc, dim=-1).to(dt), w["vc"]).reshape(B, QH * d)
             x = x + o @ w["wo"].T
-            x = x + mlp(w, rms(x, w["n2"]))
-        tok.copy_((rms(x, norm_f) @ lm_head.T).float().argmax(dim=-1))
-        pos.add_(1)
+            x = x + self.mlp(w, self.rms(x, w["n2"]))
+        self.logits.copy_((self.rms(x, self.norm_f) @ self.lm_head.T).float())
+        self.tok.copy_(self.logits.argmax(dim=-1))
+        self.pos.add_(1)
 
+    def rewind(self, tokens, tok):
+        """Undo the last ``tokens`` decoded tokens: positions and lengths go back, the input token is
+        restored.  Rows beyond the lengths are simply overwritten by the next steps."""
+        self.pos.sub_(tokens)
+        self.tok.copy_(tok)
+        for st in self.sparse:
+            st.seq_lens.sub_(tokens)
+
+
+def run_e2e(args):
+    """c5: a random-init Llama-3-8B, batch 4, 32768-token prompt prefilled densely, then greedy decoding
+    with layers 0-1 dense and layers 2.. on the sparse step (k = 655).  One decoded token for the
+    whole batch and all layers is ONE captured HIP graph; `value` is decoded tokens per second over
+    the timed replays."""
+    import torch
+
+    L = args.layers or 32
+    steps = args.steps if args.steps is not None else 512
+    warmup = args.warmup if args.warmup is not None else 8
+    B, n0, k = 4, 32768, 655
+    m = E2EModel(L=L, B=B, n0=n0, n_cap=(n0 + steps + warmup + 16 + 7) // 8 * 8, k=k)
+    prefill_s = m.prefill()
     with torch.no_grad():
-        step_body()                                                          # eager once (lazy initialisations)
+        m.step_body()                                                          # eager once (lazy initialisations)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            step_body()
+            m.step_body()
         for _ in range(warmup):
             graph.replay()
         torch.cuda.synchronize()
@@ -429,11 +465,10 @@ def run_e2e(args):
         wall_ms = (time.perf_counter() - t0) * 1e3
         gpu_ms = e0.elapsed_time(e1)
         # the sparse attention's share: a graph with only the sparse layers' launches
-        sparse = [w["st"] for w in layers if "st" in w]
         ga = torch.cuda.CUDAGraph()
         with torch.cuda.graph(ga):
-            for st in sparse:
-                st._launch(n_max, _STAGES_NO_ADVANCE)
+            for st in m.sparse:
+                st._launch(m.n_cap, _STAGES_NO_ADVANCE)
         ga.replay()
         torch.cuda.synchronize()
         a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -444,7 +479,7 @@ def run_e2e(args):
         torch.cuda.synchronize()
         attn_ms = a0.elapsed_time(a1) / 32
     ms_per_step = max(wall_ms, gpu_ms) / steps
-    lens = [int(w["st"].seq_lens[0]) for w in layers if "st" in w]
+    lens = [int(st.seq_lens[0]) for st in m.sparse]
     assert all(v == lens[0] for v in lens), "sparse layers disagree on the cache length"
     out = {
         "metric": "e2e greedy decode tokens/s (random-init Llama-3-8B, batch 4, 32k prompt)",
@@ -456,7 +491,7 @@ def run_e2e(args):
                    "graph": "one HIP graph per decoded token (all layers)"},
         "prefill_s": round(prefill_s, 2), "cache_len_after": lens[0] if lens else None,
         "sparse_attention_ms_per_step": round(attn_ms, 4),
-        "sparse_attention_us_per_layer": round(attn_ms * 1e3 / max(1, len(sparse)), 2),
+        "sparse_attention_us_per_layer": round(attn_ms * 1e3 / max(1, len(m.sparse)), 2),
         "sparse_attention_share": round(attn_ms / ms_per_step, 4),
         "roofline": None, "cpu_baseline": None,
     }
