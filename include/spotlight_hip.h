@@ -94,6 +94,20 @@ int sl_hash_mlp_pack(const void *x, const void *w1, const void *b1, const void *
                      int64_t x_stride_b, int64_t code_stride_b, int64_t code_stride_h,
                      int64_t code_stride_n, const int32_t *code_row, void *stream);
 
+/* The same hash for MANY rows per head: the codes of the keys a prompt leaves in
+ * the cache.  Replaces hash_fn(keys) + torch.sign of the whole cache
+ * (spotlight_generation.py:14-20, which the reference re-evaluates every step)
+ * followed by pack_cuda_func, evaluated once per key.
+ *   x      row (b, t) of head h at b*x_stride_b + t*x_stride_n + h*d_in  (elements)
+ *   codes  word w of (b, t, h) at b*code_stride_b + t*code_stride_n + h*code_stride_h + w
+ * Weights, layer count, widths and rounding as for sl_hash_mlp_pack, and every
+ * projection is summed in the same order: a vector gets the same code, bit for
+ * bit, from either entry point and from the decode step. */
+int sl_hash_rows_pack(const void *x, const void *w1, const void *b1, const void *w2, const void *b2,
+                      uint32_t *codes, int dtype, int n_layers, int B, int64_t n, int H, int d_in,
+                      int d_hid, int nbits, int residue, int64_t x_stride_b, int64_t x_stride_n,
+                      int64_t code_stride_b, int64_t code_stride_n, int64_t code_stride_h, void *stream);
+
 /* ---- (b) Hamming scorer -------------------------------------------------- */
 
 /* Replaces attn_k4_q28() (spotlight/kernel/attn_k4_q28.cu:100-138) and

@@ -50,6 +50,7 @@ SIGNATURES = {
     "sl_pack_sign_u32": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "sl_pack_sign_u8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p]),
     "sl_hash_mlp_pack": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_int64] * 4 + [c_void_p, c_void_p]),
+    "sl_hash_rows_pack": (c_int, [c_void_p] * 6 + [c_int, c_int, c_int, c_int64] + [c_int] * 5 + [c_int64] * 5 + [c_void_p]),
     "sl_hamming_score": (c_int, [c_void_p] * 3 + [c_int, c_int64, c_int, c_int, c_int] + [c_int64] * 3 + [c_int, c_void_p, c_void_p]),
     "sl_hamming_score_u8": (c_int, [c_void_p] * 3 + [c_int, c_int64, c_int, c_void_p]),
     "sl_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int64]),

@@ -148,6 +148,27 @@ __device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x) {
     return static_cast<uint32_t>(v);
 }
 
+// Minimum / maximum of an int over the 64 lanes of a wave; every lane receives it.  Lanes whose DPP
+// source does not exist keep their own value, which min / max absorb.
+__device__ __forceinline__ int wave_min_i32(int v) {
+    v = min(v, dpp_i32<DPP_ROW_SHR1>(v, v));
+    v = min(v, dpp_i32<DPP_ROW_SHR2>(v, v));
+    v = min(v, dpp_i32<DPP_ROW_SHR4>(v, v));
+    v = min(v, dpp_i32<DPP_ROW_SHR8>(v, v));
+    v = min(v, dpp_i32<DPP_ROW_BCAST15, 0xa>(v, v));
+    v = min(v, dpp_i32<DPP_ROW_BCAST31, 0xc>(v, v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ int wave_max_i32(int v) {
+    v = max(v, dpp_i32<DPP_ROW_SHR1>(v, v));
+    v = max(v, dpp_i32<DPP_ROW_SHR2>(v, v));
+    v = max(v, dpp_i32<DPP_ROW_SHR4>(v, v));
+    v = max(v, dpp_i32<DPP_ROW_SHR8>(v, v));
+    v = max(v, dpp_i32<DPP_ROW_BCAST15, 0xa>(v, v));
+    v = max(v, dpp_i32<DPP_ROW_BCAST31, 0xc>(v, v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

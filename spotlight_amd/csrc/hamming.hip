@@ -93,12 +93,17 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
             q_lds[e] = qb[static_cast<int64_t>(qh) * W + w];
         }
     }
+    // [lo, hi]: the score range of the workgroup's valid records (fused flavour: only these bins of its
+    // LDS histogram can be non-empty, so only they are looked at when it is flushed)
+    int *range = reinterpret_cast<int *>(hist + (FUSED ? KH * NB : 0));
     if constexpr (FUSED) {
         for (int e = tid; e < KH * NB; e += HS_THREADS) hist[e] = 0;
+        if (tid == 0) { range[0] = NB; range[1] = -1; }
     }
     if constexpr (FUSED || G_T == 0) __syncthreads();
 
     const int full = G * W * 32;
+    int s_lo = NB, s_hi = -1;
 #pragma unroll
     for (int u = 0; u < HS_U; ++u) {
         int dist = 0;
@@ -116,7 +121,11 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
         const int score = full - dist;  // matching bits
         const int64_t t = t0 + static_cast<int64_t>(u) * tok_per_pass + tl;
         if constexpr (FUSED) {
-            if (valid[u]) atomicAdd(&hist[h * NB + score], 1u);
+            if (valid[u]) {
+                atomicAdd(&hist[h * NB + score], 1u);
+                s_lo = score < s_lo ? score : s_lo;
+                s_hi = score > s_hi ? score : s_hi;
+            }
             sc_lds[h * (tok_per_pass * HS_U) + u * tok_per_pass + tl] =
                 static_cast<int16_t>(valid[u] ? score : 0);
         } else {
@@ -126,6 +135,9 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
     }
 
     if constexpr (FUSED) {
+        s_lo = wave_min_i32(s_lo);
+        s_hi = wave_max_i32(s_hi);
+        if ((tid & 63) == 0) { atomicMin(&range[0], s_lo); atomicMax(&range[1], s_hi); }
         __syncthreads();
         // head-major score rows: T int16 per head, written four at a time
         const int T = tok_per_pass * HS_U;  // a multiple of 4 (HS_THREADS * HS_U / KH, KH | 256)
@@ -145,15 +157,16 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
         // adds the non-empty ones; e / NB by multiplication (e * NB < 2^32).
         const int grp = static_cast<int>(t0 / a.hist_span) % a.hist_groups;
         uint32_t *gh = a.hist + (static_cast<int64_t>(b) * KH * a.hist_groups + grp) * NB;
-        const uint32_t inv = 0xffffffffu / static_cast<uint32_t>(NB) + 1u;
-        const int total = KH * NB;
-#pragma unroll 4
+        // bins [lo, hi] of every head: entry e = head * width + (bin - lo); e / width by
+        // multiplication (e * width < 2^32)
+        const int lo = range[0], width = range[1] - lo + 1;  // width >= 1: the workgroup holds a valid record
+        const uint32_t inv = 0xffffffffu / static_cast<uint32_t>(width) + 1u;
+        const int total = KH * width;
         for (int e = tid; e < total; e += HS_THREADS) {
-            const uint32_t c = hist[e];
-            if (c) {
-                const int hh = static_cast<int>(__umulhi(static_cast<uint32_t>(e), inv));
-                atomicAdd(&gh[static_cast<int64_t>(hh) * a.hist_groups * NB + (e - hh * NB)], c);
-            }
+            const int hh = static_cast<int>(__umulhi(static_cast<uint32_t>(e), inv));
+            const int bin = lo + (e - hh * width);
+            const uint32_t c = hist[hh * NB + bin];
+            if (c) atomicAdd(&gh[static_cast<int64_t>(hh) * a.hist_groups * NB + bin], c);
         }
     }
 }
@@ -165,7 +178,7 @@ int launch(const hamming_args &a, hipStream_t s) {
     SL_REQUIRE(blocks <= 0x7fffffffLL && a.B <= 65535, SL_ERR_UNSUPPORTED);
     size_t lds = 0;
     if (G_T == 0) lds += sizeof(uint32_t) * a.KH * a.G * W;
-    if (FUSED) lds += sizeof(uint32_t) * a.KH * a.n_bins + sizeof(int16_t) * HS_THREADS * HS_U;
+    if (FUSED) lds += sizeof(uint32_t) * (a.KH * a.n_bins + 2) + sizeof(int16_t) * HS_THREADS * HS_U;
     SL_REQUIRE(lds <= 64 * 1024, SL_ERR_UNSUPPORTED);
     hamming_kernel<W, G_T, FUSED><<<dim3(static_cast<unsigned>(blocks), a.B), dim3(HS_THREADS), lds, s>>>(a);
     return sl_check_launch();

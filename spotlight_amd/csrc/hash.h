@@ -40,3 +40,40 @@ struct hash_args {
 
 int sl_hash_launch(hash_args a, hipStream_t s);
 int sl_hash_tune(const char *key, int value);
+
+// ---- arithmetic shared by the decode-step kernel (hash.hip) and the many-rows kernel (hash_rows.hip) ----
+// Both kernels must give a vector the same code, bit for bit, whichever of them hashes it: a key
+// hashed while the prompt is prefilled and the same key hashed by a decode step are the same key.
+// They therefore share (1) the order in which the products of a projection are summed and (2) the
+// element-wise tail below.  The order, for a projection with K input rows, a partial-sum table of
+// ROWS rows (ROWS = 8 * PARTS) and K / ROWS passes:
+//     p[r]    = fma(x[r + ROWS*(P-1)], w[r + ROWS*(P-1)], ... fma(x[r], w[r], 0))        r < ROWS
+//     s[part] = (((0 + p[8 part]) + p[8 part + 1]) + ...) + p[8 part + 7]               part < PARTS
+//     total   = ((0 + s[0]) + s[1]) + ... + s[PARTS - 1]
+// first projection: ROWS = 4096 / d_hid; second projection: ROWS = 32.
+
+__device__ __forceinline__ float hash_silu(float x) { return x / (1.0f + expf(-x)); }
+
+// value of hidden / output column `col` after the first projection's sum `total`: rounded to T where the
+// torch expression of the reference materialises a tensor (matmul, bias add, SiLU, residual add)
+template <typename T, int NL>
+__device__ __forceinline__ float hash_finish_l1(float total, bool has_bias, float bias, bool residue, float x_col) {
+    float v = round_to<T>(total);
+    if (has_bias) v = round_to<T>(v + bias);
+    if constexpr (NL == 2) v = round_to<T>(hash_silu(v));
+    if (residue) v = round_to<T>(v + x_col);
+    return v;
+}
+
+template <typename T>
+__device__ __forceinline__ float hash_finish_l2(float total, bool has_bias, float bias, bool residue, float hid_col) {
+    float v = round_to<T>(total);
+    if (has_bias) v = round_to<T>(v + bias);
+    if (residue) v = round_to<T>(v + hid_col);
+    return v;
+}
+
+int sl_hash_rows_launch(const void *x, const void *w1, const void *b1, const void *w2, const void *b2, uint32_t *codes,
+                        int dtype, int n_layers, int B, int64_t n, int H, int d_in, int d_hid, int nbits, int residue,
+                        int64_t x_stride_b, int64_t x_stride_n, int64_t code_stride_b, int64_t code_stride_n,
+                        int64_t code_stride_h, hipStream_t s);

@@ -38,8 +38,6 @@ __device__ __forceinline__ bool sl_aligned_dev(const void *p, uintptr_t a) {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
 }
 
-__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
-
 template <int D_HID> struct l1_shape {
     static constexpr int LPR = D_HID / 8;             // lanes per weight row
     static constexpr int RPP = HK_THREADS / LPR;      // rows per pass
@@ -240,15 +238,8 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     if (tid < D_HID) {
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
-            float v = round_to<T>(v1[rr]);
-            if (sd.b1) v = round_to<T>(v + bias1);
-            if constexpr (NL == 2) {
-                v = round_to<T>(silu_f32(v));
-                if (a.residue) v = round_to<T>(v + xs[rr][tid]);
-                hidl[rr][tid] = v;
-            } else {
-                if (a.residue) v = round_to<T>(v + xs[rr][tid]);
-            }
+            const float v = hash_finish_l1<T, NL>(v1[rr], sd.b1 != nullptr, bias1, a.residue != 0, xs[rr][tid & (HK_DIN - 1)]);
+            if constexpr (NL == 2) hidl[rr][tid] = v;
             v1[rr] = v;
         }
     }
@@ -285,12 +276,8 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
         fold_columns<HK_NBITS, R>(red, sub, pre);
         if (tid < HK_NBITS) {
 #pragma unroll
-            for (int rr = 0; rr < R; ++rr) {
-                float v = round_to<T>(pre[rr]);
-                if (sd.b2) v = round_to<T>(v + bias2);
-                if (a.residue) v = round_to<T>(v + hidl[rr][tid]);
-                pre[rr] = v;
-            }
+            for (int rr = 0; rr < R; ++rr)
+                pre[rr] = hash_finish_l2<T>(pre[rr], sd.b2 != nullptr, bias2, a.residue != 0, hidl[rr][tid & (D_HID - 1)]);
         }
     }
     // sign bits: the waves that hold the nbits pre-activations ballot 64 bits each

@@ -65,29 +65,12 @@ class HashWeights:
         """Gaussian projection, not orthogonalised (linearhashing_generation.py:227)."""
         return HashWeights(torch.randn(H, d, nbits, generator=generator).to(dtype).to(device))
 
-    def hash_rows(self, x: torch.Tensor) -> torch.Tensor:
+    def hash_rows(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Codes of many rows per head (prefill): x [B,n,H,d] -> uint32 [B,n,H,nbits/32].
 
-        Library GEMMs for the projections (this is GEMM-shaped work), then the
-        HIP pack kernel; rounding follows the reference's torch expression."""
-        B, n, H, d = x.shape
-        h = x.permute(2, 0, 1, 3).reshape(H, B * n, d)
-        y = torch.bmm(h, self.w1)
-        if self.b1 is not None:
-            y = y + self.b1[:, None, :]
-        if self.w2 is not None:
-            y = torch.nn.functional.silu(y)
-            if self.residue:
-                y = y + h
-            z = torch.bmm(y, self.w2)
-            if self.b2 is not None:
-                z = z + self.b2[:, None, :]
-            if self.residue:
-                z = z + y
-        else:
-            z = y + h if self.residue else y
-        z = z.reshape(H, B, n, -1).permute(1, 2, 0, 3).contiguous()
-        return K.pack_cuda_func(z)
+        The HIP kernel for many rows; it sums exactly as the decode step's hash does, so a key
+        gets the same code whether it arrives with the prompt or as a decoded token."""
+        return K.hash_rows_pack(x, self.w1, self.b1, self.w2, self.b2, self.residue, out=out)
 
 
 class LayerDecodeState:

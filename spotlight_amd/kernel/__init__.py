@@ -316,6 +316,32 @@ def hash_mlp_pack(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor],
     return codes
 
 
+def hash_rows_pack(x: torch.Tensor, w1: torch.Tensor, b1: Optional[torch.Tensor],
+                   w2: Optional[torch.Tensor] = None, b2: Optional[torch.Tensor] = None,
+                   residue: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same hash for many rows per head: x [B,n,H,d_in] -> uint32 [B,n,H,nbits/32] (or into
+    ``out``, any tensor of that shape whose last dimension is contiguous, e.g. a slice of a cache).
+    Bit-identical to ``hash_mlp_pack`` row by row: both sum the projections in one order."""
+    _need_gpu(x, w1)
+    B, n, H, d_in = x.shape
+    d_hid = w1.shape[2]
+    n_layers = 2 if w2 is not None else 1
+    nbits = w2.shape[2] if w2 is not None else d_hid
+    assert x.stride(3) == 1 and x.stride(2) == d_in, "rows of a head must be contiguous, heads adjacent"
+    for t in (w1, b1, w2, b2):
+        assert t is None or (t.is_contiguous() and t.dtype == x.dtype)
+    if out is None:
+        out = torch.empty((B, n, H, nbits // 32), dtype=torch.uint32, device=x.device)
+    assert out.shape == (B, n, H, nbits // 32) and out.dtype == torch.uint32 and out.stride(3) == 1
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    with torch.cuda.device(x.device):
+        _lib.check(_L.sl_hash_rows_pack(
+            x.data_ptr(), w1.data_ptr(), ptr(b1), ptr(w2), ptr(b2), out.data_ptr(), _dtype(x), n_layers,
+            B, n, H, d_in, d_hid, nbits, int(residue), x.stride(0), x.stride(1),
+            out.stride(0), out.stride(1), out.stride(2), _stream()), "sl_hash_rows_pack")
+    return out
+
+
 def cache_append(dst: torch.Tensor, src: torch.Tensor, start: int = 0,
                  seq_lens: Optional[torch.Tensor] = None) -> None:
     """dst[b, start + seq_lens[b] : ... + t] = src[b]  for dst [B,L,...] and
