@@ -44,7 +44,10 @@ typedef enum { SL_HEADMAP_INTERLEAVED = 0, SL_HEADMAP_BLOCKED = 1 } sl_head_map;
 const char *sl_strerror(int status);
 int sl_version(void);
 
-/* Process-wide launch heuristics (host memory, not thread safe).  Keys:
+/* Process-wide launch heuristics: a debugging and benchmarking aid, NOT part of
+ * the re-entrancy contract above (host memory, not thread safe; change them
+ * only while no other thread is inside the library).  The defaults are what
+ * every documented figure was measured with.  Keys:
  * "attn_target_wgs": workgroups the attention launch aims for (default 256);
  * it decides into how many runs the selected rows of a (b, kv head) are cut;
  * "fuse_select_attend": 1 (default) lets the decode step run selection and

@@ -44,13 +44,17 @@ class KVHash:
         return self.key_cache[layer_idx][:, :end]
 
 
+MAX_SCORE_BOUND = 4607   # the largest score sl_topk_select covers (36 query heads of 128 bits per kv head)
+
+
 def topk_and_gather(attn, keys, vals, budget, max_score: Optional[int] = None):
     """attn int16 [B,n,KH] scores, keys/vals [B,L,KH,d] -> (K_sel, V_sel) [B,budget,KH,d].
 
-    ``max_score`` bounds the scores (G * nbits for the Hamming scorer); when it
-    is not given it is read back from ``attn`` (one device sync)."""
+    ``max_score`` bounds the scores (G * nbits for the Hamming scorer).  Without it the widest
+    range the selector covers is assumed (scores up to 4607): still exact, never a device
+    round trip, but more histogram bins than a known bound needs."""
     if max_score is None:
-        max_score = int(attn.max().item()) if attn.numel() else 0
+        max_score = MAX_SCORE_BOUND
     ind = K.topk_select(attn, budget, max_score)
     return K.gather_kv(keys, vals, ind)
 
@@ -63,6 +67,7 @@ class KVCache:
     def __init__(self, batch_size, num_kv_heads, head_dim, num_layers, dtype=torch.bfloat16, device=None,
                  **kwargs):
         self.num_kv_heads = num_kv_heads
+        self.max_score = kwargs.get("max_score")   # optional bound of the scores gather() will see (G * nbits)
         self.length = [0 for _ in range(num_layers)]
         self.max_length = self.init_seq_length
         self.num_layers = num_layers
@@ -76,7 +81,7 @@ class KVCache:
     def gather(self, layer_idx, attn, budget, max_score: Optional[int] = None):
         n = attn.shape[1]
         return topk_and_gather(attn, self.key_cache[layer_idx][:, :n], self.val_cache[layer_idx][:, :n],
-                               budget, max_score)
+                               budget, max_score if max_score is not None else self.max_score)
 
     def update(self, layer_idx, key, val):
         start = self.length[layer_idx]
