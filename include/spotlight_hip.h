@@ -57,6 +57,8 @@ int sl_version(void);
  * (1, 2 or 4; 0 = by batch size, the default);
  * "attn_wide_rows": rows per run from which the attention launch uses 8 waves per
  * workgroup instead of 4 (default 128);
+ * "attn_mfma": 1 puts the q.K products of the attention on the matrix cores
+ * (16-bit inputs; default 0: packed dot products and a lane butterfly);
  * "hist_copies": copies of the score histogram (4, 8, 16 or 32; 0 = by cache
  * length), to be set before any workspace is sized. */
 int sl_tune(const char *key, int value);

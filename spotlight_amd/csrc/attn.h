@@ -28,3 +28,4 @@ size_t sl_attn_ws_bytes(int B, int QH, int KH, int k);
 int sl_attn_prepare(attn_args &a, void *ws, size_t ws_bytes);
 int sl_attn_launch(attn_args a, void *ws, size_t ws_bytes, hipStream_t s);
 int sl_attn_tune(const char *key, int value);
+bool sl_attn_use_mfma();  // sl_tune("attn_mfma", 1): 16-bit inputs score on the matrix cores

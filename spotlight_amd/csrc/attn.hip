@@ -22,12 +22,12 @@ constexpr int AT_MAX_ROWS = 1024;    // rows per run (LDS row-number buffer)
 // the only part that has to stay zero between calls.
 constexpr size_t AT_COUNTER_BYTES = 64 * 1024;
 
-template <typename T, int G, int NW, bool FETCH>
+template <typename T, int G, int NW, bool FETCH, bool MF>
 __global__ __launch_bounds__(NW * 64) void sparse_attn_kernel(attn_args a) {
     constexpr int AT_THREADS = NW * 64;
     __shared__ int s_row[AT_MAX_ROWS];
     __shared__ int s_src[FETCH ? AT_MAX_ROWS : 1];
-    __shared__ attn_shared<G, NW> sh;
+    __shared__ attn_shared<G, NW, MF> sh;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int r_lo = split * a.rows;
     const int r_hi = r_lo + a.rows < a.k ? r_lo + a.rows : a.k;
@@ -38,24 +38,33 @@ __global__ __launch_bounds__(NW * 64) void sparse_attn_kernel(attn_args a) {
         for (int i = threadIdx.x; i < a.rows; i += AT_THREADS) s_src[i] = r_lo + i < r_hi ? fetch[r_lo + i] : -1;
     }
     __syncthreads();
-    attend_rows_and_merge<T, G, NW, FETCH>(a, b, h, split, gridDim.x, s_row, a.rows, sh, s_src);
+    attend_rows_and_merge<T, G, NW, FETCH, MF>(a, b, h, split, gridDim.x, s_row, a.rows, sh, s_src);
 }
 
 int g_attn_wide_rows = AT_WIDE_ROWS;  // sl_tune("attn_wide_rows", n)
+int g_attn_mfma = 0;                  // sl_tune("attn_mfma", 0 | 1): score phase on the matrix cores (16-bit inputs)
 
-template <typename T, int G>
-int launch(const attn_args &a, hipStream_t s) {
+template <typename T, int G, bool MF>
+int launch_mf(const attn_args &a, hipStream_t s) {
     const int S = (a.k + a.rows - 1) / a.rows;
     const dim3 grid(S, a.KH, a.B);
     const bool wide = a.rows >= g_attn_wide_rows;
     if (a.fetch) {
-        if (wide) sparse_attn_kernel<T, G, 8, true><<<grid, dim3(512), 0, s>>>(a);
-        else sparse_attn_kernel<T, G, 4, true><<<grid, dim3(256), 0, s>>>(a);
+        if (wide) sparse_attn_kernel<T, G, 8, true, MF><<<grid, dim3(512), 0, s>>>(a);
+        else sparse_attn_kernel<T, G, 4, true, MF><<<grid, dim3(256), 0, s>>>(a);
     } else {
-        if (wide) sparse_attn_kernel<T, G, 8, false><<<grid, dim3(512), 0, s>>>(a);
-        else sparse_attn_kernel<T, G, 4, false><<<grid, dim3(256), 0, s>>>(a);
+        if (wide) sparse_attn_kernel<T, G, 8, false, MF><<<grid, dim3(512), 0, s>>>(a);
+        else sparse_attn_kernel<T, G, 4, false, MF><<<grid, dim3(256), 0, s>>>(a);
     }
     return sl_check_launch();
+}
+
+template <typename T, int G>
+int launch(const attn_args &a, hipStream_t s) {
+    if constexpr (sizeof(T) == 2) {
+        if (g_attn_mfma) return launch_mf<T, G, true>(a, s);
+    }
+    return launch_mf<T, G, false>(a, s);
 }
 
 template <typename T>
@@ -92,8 +101,11 @@ int pick_rows(int B, int KH, int k) {
 int sl_attn_tune(const char *key, int value) {
     if (!strcmp(key, "attn_target_wgs") && value > 0) { g_attn_target_wgs = value; return SL_OK; }
     if (!strcmp(key, "attn_wide_rows") && value > 0) { g_attn_wide_rows = value; return SL_OK; }
+    if (!strcmp(key, "attn_mfma") && (value == 0 || value == 1)) { g_attn_mfma = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
+
+bool sl_attn_use_mfma() { return g_attn_mfma != 0; }
 
 size_t sl_attn_ws_bytes(int B, int QH, int KH, int k) {
     if (B <= 0 || QH <= 0 || KH <= 0 || k <= 0) return 0;

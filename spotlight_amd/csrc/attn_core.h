@@ -43,9 +43,10 @@ template <int G> struct attn_shape {
     static constexpr int U = 16 / GP;                       // rows a 16-lane group scores per chunk
 };
 
-template <int G, int NW>
+template <int G, int NW, bool MF = false>
 struct attn_shared {
-    static constexpr int GP = attn_shape<G>::GP, U = attn_shape<G>::U;
+    static constexpr int GP = attn_shape<G>::GP;
+    static constexpr int U = MF ? 4 : attn_shape<G>::U;  // matrix-core flavour: a wave scores a 16-row tile
     static constexpr int NLG = NW * 4;    // 16-lane groups in the workgroup
     static constexpr int CH = NLG * U;    // rows per chunk
     static constexpr int RW = CH / NW;    // rows of a chunk one wave accumulates
@@ -108,6 +109,24 @@ template <typename T> __device__ __forceinline__ float dot_slice8(const slice8<T
         return dot2_acc<T>(a.w.w, b.w.w, d);
     }
 }
+
+// ---- matrix-core flavour of the score phase (16-bit inputs) -----------------------------------------
+// S[16 rows][16 heads] = K[16][128] . Q^T[128][16] as four v_mfma_f32_16x16x32: lane (m = lane % 16,
+// kb = lane / 16) holds elements 32 kb .. 32 kb + 31 of K row m (four 16-byte loads; operand A) and of
+// query head m (operand B, heads >= G are zero); instruction j consumes elements 32 kb + 8 j .. + 7 of
+// both.  The result has head lane % 16 of rows 4 (lane / 16) .. + 3 in the lane's four accumulators.
+typedef __bf16 sl_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 sl_f16x8 __attribute__((ext_vector_type(8)));
+typedef float sl_f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> __device__ __forceinline__ sl_f32x4 mfma_16x16x32(const uint4 &a, const uint4 &b, sl_f32x4 c);
+template <> __device__ __forceinline__ sl_f32x4 mfma_16x16x32<bf16_t>(const uint4 &a, const uint4 &b, sl_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sl_bf16x8, a), __builtin_bit_cast(sl_bf16x8, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ sl_f32x4 mfma_16x16x32<f16_t>(const uint4 &a, const uint4 &b, sl_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(sl_f16x8, a), __builtin_bit_cast(sl_f16x8, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ sl_f32x4 mfma_16x16x32<float>(const uint4 &, const uint4 &, sl_f32x4 c) { return c; }
 
 // Two consecutive elements as loaded, and as fp32.
 template <typename T> struct pair_raw { uint32_t w; };
@@ -189,11 +208,12 @@ template <int U> __device__ __forceinline__ float head_max(float v) {
 // s_src[i] >= 0 names a row of the source store that row s_row[i] is to be filled
 // from: the kernel reads that row instead, and writes the K slices / V pairs it
 // loaded to row s_row[i] of keys / vals after it has used them.
-template <typename T, int G, int NW, bool FETCH = false>
+template <typename T, int G, int NW, bool FETCH = false, bool MF = false>
 __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b, int h, int split, int S,
-                                                      const int *s_row, int n_rows, attn_shared<G, NW> &sh,
+                                                      const int *s_row, int n_rows, attn_shared<G, NW, MF> &sh,
                                                       const int *s_src = nullptr) {
-    using SH = attn_shared<G, NW>;
+    static_assert(!MF || sizeof(T) == 2, "the matrix-core flavour takes 16-bit inputs");
+    using SH = attn_shared<G, NW, MF>;
     constexpr int NT = NW * 64, NLG = SH::NLG, GP = SH::GP, U = SH::U, CH = SH::CH, RW = SH::RW;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -206,14 +226,24 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
     slice8<T> qs[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) qs[g] = load_slice8<T>(qb + g * AT_D);
+    uint4 qf[4];   // matrix-core flavour: elements 32 kb .. + 31 of query head (lane % 16), zero beyond G
+    if constexpr (MF) {
+        const T *qm = static_cast<const T *>(a.q) + static_cast<int64_t>(b) * a.q_stride_b +
+                      (static_cast<int64_t>(h) * G + (sub < G ? sub : 0)) * AT_D + (lane >> 4) * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            qf[j] = reinterpret_cast<const uint4 *>(qm)[j];
+            if (sub >= G) qf[j] = make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
     const T *kb = static_cast<const T *>(a.keys) + static_cast<int64_t>(b) * a.kv_stride_b +
-                  static_cast<int64_t>(h) * a.kv_stride_h + sub * 8;
+                  static_cast<int64_t>(h) * a.kv_stride_h + (MF ? (lane >> 4) * 32 : sub * 8);
     const T *vb = static_cast<const T *>(a.vals) + static_cast<int64_t>(b) * a.kv_stride_b +
                   static_cast<int64_t>(h) * a.kv_stride_h + lane * 2;
     const T *skb = nullptr, *svb = nullptr;
     if constexpr (FETCH) {
         skb = static_cast<const T *>(a.src_keys) + static_cast<int64_t>(b) * a.src_stride_b +
-              static_cast<int64_t>(h) * a.src_stride_h + sub * 8;
+              static_cast<int64_t>(h) * a.src_stride_h + (MF ? (lane >> 4) * 32 : sub * 8);
         svb = static_cast<const T *>(a.src_vals) + static_cast<int64_t>(b) * a.src_stride_b +
               static_cast<int64_t>(h) * a.src_stride_h + lane * 2;
     }
@@ -228,19 +258,31 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         // every load of the chunk first: U key slices for the score phase, RW value
         // pairs for the accumulation phase (an absent or skipped row re-reads row 0
         // and gets probability 0): no branch sits between the loads
-        int row[U], src[U];
-        slice8<T> ks[U];
+        constexpr int KU = MF ? 1 : U, KS = MF ? 4 : 1;
+        int row[KU], src[KU];
+        slice8<T> ks[KU];   // dot flavour: one 8-element slice of U rows
+        uint4 kf[KS];       // matrix-core flavour: 32 elements of ONE row (row base + 16 wave + lane % 16 of the chunk)
+        if constexpr (MF) {
+            const int ri = base + wave * 16 + sub;
+            row[0] = ri < n_rows ? s_row[ri] : -1;
+            src[0] = FETCH && ri < n_rows && row[0] >= 0 ? s_src[ri] : -1;
+            const T *p = kb + static_cast<int64_t>(row[0] >= 0 ? row[0] : 0) * a.kv_stride_n;
+            if constexpr (FETCH) p = src[0] >= 0 ? skb + static_cast<int64_t>(src[0]) * a.src_stride_n : p;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int ri = base + u * NLG + rslot;
-            row[u] = ri < n_rows ? s_row[ri] : -1;
-            src[u] = FETCH && ri < n_rows && row[u] >= 0 ? s_src[ri] : -1;
-        }
+            for (int j = 0; j < 4; ++j) kf[j] = reinterpret_cast<const uint4 *>(p)[j];
+        } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const T *p = kb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n;
-            if constexpr (FETCH) p = src[u] >= 0 ? skb + static_cast<int64_t>(src[u]) * a.src_stride_n : p;
-            ks[u] = load_slice8<T>(p);
+            for (int u = 0; u < U; ++u) {
+                const int ri = base + u * NLG + rslot;
+                row[u] = ri < n_rows ? s_row[ri] : -1;
+                src[u] = FETCH && ri < n_rows && row[u] >= 0 ? s_src[ri] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const T *p = kb + static_cast<int64_t>(row[u] >= 0 ? row[u] : 0) * a.kv_stride_n;
+                if constexpr (FETCH) p = src[u] >= 0 ? skb + static_cast<int64_t>(src[u]) * a.src_stride_n : p;
+                ks[u] = load_slice8<T>(p);
+            }
         }
         pair_raw<T> vs[RW];
         int vrow[RW], vsrc[RW];
@@ -257,29 +299,57 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             vs[j] = load_pair<T>(p);
         }
 
-        // scores: partial dot products of this lane's slice, then the butterfly
-        float part[16];
+        // scores.  Dot flavour: partial dot products of this lane's slice, then the butterfly: ONE
+        // score per lane.  Matrix-core flavour: four instructions leave FOUR scores per lane (head
+        // lane % 16 of the rows 4 (lane / 16) .. + 3 of the wave's tile).
+        constexpr int NS = MF ? 4 : 1;
+        float sc[NS];
+        bool valid[NS];
+        const int my_head = MF ? sub : g_l;
+        if constexpr (MF) {
+            sl_f32x4 d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int g = i / U, u = i % U;
-            part[i] = g < G ? dot_slice8<T>(qs[g < G ? g : 0], ks[u]) : 0.f;
+            for (int j = 0; j < 4; ++j) d = mfma_16x16x32<T>(kf[j], qf[j], d);
+            if constexpr (FETCH) {
+                if (src[0] >= 0) {
+                    T *dst = const_cast<T *>(kb) + static_cast<int64_t>(row[0]) * a.kv_stride_n;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) reinterpret_cast<uint4 *>(dst)[j] = kf[j];
+                }
+            }
+            const int r0 = base + wave * 16 + (lane >> 4) * 4;   // the lane's four result rows
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                valid[r] = r0 + r < n_rows && s_row[r0 + r < n_rows ? r0 + r : 0] >= 0 && sub < G;
+                sc[r] = valid[r] ? d[r] * a.scale : -INFINITY;
+            }
+            float wm = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            wm = fmaxf(wm, __shfl_xor(wm, 16, 64));
+            wm = fmaxf(wm, __shfl_xor(wm, 32, 64));
+            if (lane < 16 && sub < GP) sh.wmax[wave][sub] = wm;
+        } else {
+            float part[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int g = i / U, u = i % U;
+                part[i] = g < G ? dot_slice8<T>(qs[g < G ? g : 0], ks[u]) : 0.f;
+            }
+            float s = row16_transpose_sum(part, sub) * a.scale;
+            if constexpr (FETCH) {
+                // the fetched K slices have been used (and therefore waited for): put them in their rows
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (src[u] >= 0) store_slice8<T>(const_cast<T *>(kb) + static_cast<int64_t>(row[u]) * a.kv_stride_n, ks[u]);
+            }
+            int my_row = row[0];
+#pragma unroll
+            for (int u = 1; u < U; ++u) my_row = u_l == u ? row[u] : my_row;
+            valid[0] = my_row >= 0 && g_l < G;
+            sc[0] = valid[0] ? s : -INFINITY;
+            // chunk maximum per head: in the wave, then over the waves through LDS
+            const float wm = head_max<U>(sc[0]);
+            if (lane < 16 && u_l == 0) sh.wmax[wave][g_l] = wm;
         }
-        float s = row16_transpose_sum(part, sub) * a.scale;
-        if constexpr (FETCH) {
-            // the fetched K slices have been used (and therefore waited for): put them in their rows
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (src[u] >= 0) store_slice8<T>(const_cast<T *>(kb) + static_cast<int64_t>(row[u]) * a.kv_stride_n, ks[u]);
-        }
-        int my_row = row[0];
-#pragma unroll
-        for (int u = 1; u < U; ++u) my_row = u_l == u ? row[u] : my_row;
-        const bool valid = my_row >= 0 && g_l < G;
-        s = valid ? s : -INFINITY;
-
-        // chunk maximum per head: in the wave, then over the waves through LDS
-        const float wm = head_max<U>(s);
-        if (lane < 16 && u_l == 0) sh.wmax[wave][g_l] = wm;
         __syncthreads();
         float m_new[GP];
 #pragma unroll
@@ -290,9 +360,16 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             for (int g = 0; g < GP; ++g) m_new[g] = fmaxf(m_new[g], sh.wmax[w][g]);
         float my_m = m_new[0];
 #pragma unroll
-        for (int g = 1; g < GP; ++g) my_m = g_l == g ? m_new[g] : my_m;
-        const float p = valid ? __expf(s - my_m) : 0.f;  // a valid score makes my_m finite
-        sh.p[u_l * NLG + rslot][g_l] = p;
+        for (int g = 1; g < GP; ++g) my_m = my_head == g ? m_new[g] : my_m;
+        if constexpr (MF) {
+            if (sub < GP) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)   // a valid score makes my_m finite
+                    sh.p[wave * 16 + (lane >> 4) * 4 + r][sub] = valid[r] ? __expf(sc[r] - my_m) : 0.f;
+            }
+        } else {
+            sh.p[u_l * NLG + rslot][g_l] = valid[0] ? __expf(sc[0] - my_m) : 0.f;
+        }
         __syncthreads();
 
         // values: rescale what earlier chunks left (exp(-inf) = 0 on the first), then

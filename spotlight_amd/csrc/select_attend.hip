@@ -27,12 +27,12 @@ template <bool dummy = true> struct sa_static_checks {
     static_assert(SA_MAX_BLOCKS == AT_MAX_SPLITS, "one attention run per token block");
 };
 
-template <typename T, int G, int NG>
+template <typename T, int G, int NG, bool MF>
 __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args sa, attn_args aa) {
     __shared__ uint32_t s_wave[64];  // [0,32): scans, [32,64): block_sum2
     __shared__ int s_tn[4];
     __shared__ int32_t s_list[SA_BLOCK];
-    __shared__ attn_shared<G, SA_NW> sh;
+    __shared__ attn_shared<G, SA_NW, MF> sh;
 
     const int tid = threadIdx.x;
     const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -63,15 +63,23 @@ __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args s
     // the list goes out with coalesced stores; the attention then runs over it
     __syncthreads();
     for (int i = tid; i < n_kept; i += SA_THREADS) out[first + i] = s_list[i];
-    attend_rows_and_merge<T, G, SA_NW>(aa, b, h, blk, S, s_list, n_kept, sh);
+    attend_rows_and_merge<T, G, SA_NW, false, MF>(aa, b, h, blk, S, s_list, n_kept, sh);
+}
+
+template <typename T, int G, bool MF>
+int launch_mf(const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
+    if (sa.hist_groups == 16) select_attend_kernel<T, G, 16, MF><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
+    else if (sa.hist_groups == 8) select_attend_kernel<T, G, 8, MF><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
+    else select_attend_kernel<T, G, 4, MF><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
+    return sl_check_launch();
 }
 
 template <typename T, int G>
 int launch_ng(const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
-    if (sa.hist_groups == 16) select_attend_kernel<T, G, 16><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
-    else if (sa.hist_groups == 8) select_attend_kernel<T, G, 8><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
-    else select_attend_kernel<T, G, 4><<<grid, dim3(SA_THREADS), 0, s>>>(sa, aa);
-    return sl_check_launch();
+    if constexpr (sizeof(T) == 2) {
+        if (sl_attn_use_mfma()) return launch_mf<T, G, true>(sa, aa, grid, s);
+    }
+    return launch_mf<T, G, false>(sa, aa, grid, s);
 }
 
 template <typename T>

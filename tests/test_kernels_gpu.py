@@ -253,6 +253,24 @@ def test_sparse_attention(K, B, QH, KH, L, k, dtype):
     assert np.abs(got - want).max() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("B,QH,KH,L,k", ATTN_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_sparse_attention_matrix_core_flavour(K, B, QH, KH, L, k, dtype):
+    """The same attention with the q.K products on the matrix cores (sl_tune "attn_mfma")."""
+    from spotlight_amd import _lib
+    L_ = _lib.load()
+    q, keys, vals, idx = _attn_inputs(_gen(L + k), B, QH, KH, L, k, dtype)
+    if k > 1:
+        idx[:, :, k // 2] = -1                  # a skipped row in the middle
+    _lib.check(L_.sl_tune(b"attn_mfma", 1), "sl_tune")
+    try:
+        got = K.sparse_gqa_attn(q.to(DEV), keys.to(DEV), vals.to(DEV), idx.to(DEV)).float().cpu().numpy()
+    finally:
+        _lib.check(L_.sl_tune(b"attn_mfma", 0), "sl_tune")
+    want = orc.sparse_attention(q.float().numpy(), keys.float().numpy(), vals.float().numpy(), idx.numpy())
+    assert np.abs(got - want).max() <= TOL[dtype]
+
+
 def test_sparse_attention_skips_negative_rows_and_head_major(K):
     q, keys, vals, idx = _attn_inputs(_gen(21), 2, 32, 8, 400, 50, torch.float32)
     idx[:, :, 40:] = -1
