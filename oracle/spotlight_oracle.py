@@ -21,6 +21,10 @@ the reference checkout) and how it is pinned without running the reference:
   sparse_attention               textbook softmax in fp64, equivalence with the
                                  reference's masked dense form on small n
   mlp_hash / linear_hash         textbook batched matmul + SiLU in fp64
+  apply_rope                     the same rotation written with complex numbers
+  reference_self_attn_forward,   tests/test_oracle_composite.py: textbook RoPE as a
+  decode_step_reference_form,    complex rotation, attention as fp64 loops over the
+  decode_step_cached_codes       GQA groups, selection as a brute force on packed codes
   CacheModel                     slice assignment
   LruModel                       PARITY UNPINNED by the reference (there is no
                                  LRU in it): pinned only by its own sequential
