@@ -469,8 +469,9 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         const int g = (e < G * AT_D ? e : 0) / AT_D, c = e % AT_D;
 #pragma unroll
         for (int sp = 0; sp < AT_MAX_SPLITS; ++sp) {
-            const float v = ld_agent(pb + (static_cast<int64_t>(sp < S ? sp : 0) * G + g) * AT_PART + c);
-            pa[i][sp] = (e < G * AT_D && sp < S) ? v : 0.f;
+            float v = 0.f;
+            if (sp < S) v = ld_agent(pb + (static_cast<int64_t>(sp) * G + g) * AT_PART + c);  // uniform: absent runs cost nothing
+            pa[i][sp] = e < G * AT_D ? v : 0.f;
         }
     }
     static_assert(AT_MAX_SPLITS == 16, "the runs of a head fit one 16-lane row");

@@ -192,8 +192,12 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     select_args ta{};
     ta.B = p.B; ta.KH = p.KH; ta.n_bins = G * p.nbits + 1;
     sl_select_carve(ta, ws + L.select, p.n_cap);
-    ha.zero_words = ta.hist;  // the scorer of this step starts from a clean histogram
-    ha.zero_count = static_cast<int64_t>(p.B) * p.KH * ta.n_bins * ta.hist_groups;
+    ta.hist_used = sl_select_hist_used(ta, p.n_max);
+    // the scorer of this step starts from a clean histogram: per (b, kv head) the copies this launch can reach
+    ha.zero_words = ta.hist;
+    ha.zero_rows = p.B * p.KH;
+    ha.zero_count = static_cast<int64_t>(ta.n_bins) * ta.hist_used;
+    ha.zero_stride = static_cast<int64_t>(ta.n_bins) * ta.hist_groups;
     ha.len_out = n_rows;
     // 2. score seq_lens[b] + 1 rows
     hamming_args sa{};

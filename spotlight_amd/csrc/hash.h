@@ -26,8 +26,11 @@ struct hash_args {
     hash_side side[2];
     int n_sides;
     int dtype, n_layers, B, d_in, d_hid, nbits, residue;
-    uint32_t *zero_words;  // optional: words the launch also clears (next step's histogram)
-    int64_t zero_count;
+    // optional: words the launch also clears (next step's histogram): zero_rows runs of zero_count
+    // words each, zero_stride words apart
+    uint32_t *zero_words;
+    int64_t zero_count, zero_stride;
+    int zero_rows;
     // optional [B]: receives code_row[b] + 1 of the last side, i.e. the number of cached rows once this
     // launch's row is appended.  Later launches of the step read lengths from here, so that no launch
     // reads a length another workgroup of the same launch advances.

@@ -164,15 +164,20 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     const uint4 cp0 = reinterpret_cast<const uint4 *>(src0 + cp_off)[cp_c];
     const uint4 cp1 = reinterpret_cast<const uint4 *>(src1 + cp_off)[cp_c];
 
-    // housekeeping that rides along: clear the next score histogram
+    // housekeeping that rides along: clear the next score histogram (zero_rows runs of zero_count words)
     if (a.zero_words) {
         const int64_t n_wg = static_cast<int64_t>(gridDim.x) * gridDim.y;
         const int64_t wg = static_cast<int64_t>(blockIdx.y) * gridDim.x + blockIdx.x;
         // 16 bytes per store while whole quads remain, single words for the tail
-        uint4 *z4 = reinterpret_cast<uint4 *>(a.zero_words);
-        const int64_t n4 = sl_aligned_dev(a.zero_words, 16) ? a.zero_count / 4 : 0;
-        for (int64_t i = wg * HK_THREADS + tid; i < n4; i += n_wg * HK_THREADS) z4[i] = make_uint4(0u, 0u, 0u, 0u);
-        for (int64_t i = n4 * 4 + wg * HK_THREADS + tid; i < a.zero_count; i += n_wg * HK_THREADS) a.zero_words[i] = 0u;
+        const bool quads = sl_aligned_dev(a.zero_words, 16) && a.zero_stride % 4 == 0;
+        const int64_t n4 = quads ? a.zero_count / 4 : 0, per_row = n4 + (a.zero_count - n4 * 4);
+        const int64_t total = per_row * a.zero_rows;
+        for (int64_t i = wg * HK_THREADS + tid; i < total; i += n_wg * HK_THREADS) {
+            const int64_t row = i / per_row, e = i - row * per_row;
+            uint32_t *base = a.zero_words + row * a.zero_stride;
+            if (e < n4) reinterpret_cast<uint4 *>(base)[e] = make_uint4(0u, 0u, 0u, 0u);
+            else base[n4 * 4 + (e - n4)] = 0u;
+        }
     }
 
     float xrow[4] = {x0, x1, x2, x3};

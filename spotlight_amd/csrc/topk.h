@@ -10,6 +10,7 @@ struct select_args {
     uint32_t *hist;           // [B, KH, hist_groups, n_bins]: the copies are summed
     int hist_groups;          // 4, 8, 16 or 32
     int hist_span;            // token t is counted into copy (t / hist_span) % hist_groups
+    int hist_used;            // copies that can hold counts for this launch's n tokens: the others are not read
     int32_t *thr_need;        // [B, KH, 2] scratch: threshold bin, tokens to take from it
     uint32_t *block_cnt;      // [B, KH, n_blocks] scratch: (above | equal << 16) per token block
     int n_blocks;             // row length of block_cnt
@@ -25,5 +26,6 @@ int64_t sl_select_hist_span(int64_t n);
 size_t sl_select_ws_bytes(int B, int KH, int n_bins, int64_t n);
 // points hist / thr_need / block_cnt of `a` into `ws` (a.B, a.KH, a.n_bins set)
 void sl_select_carve(select_args &a, void *ws, int64_t n_for_blocks);
+int sl_select_hist_used(const select_args &a, int64_t n);
 int sl_select_launch(const select_args &a, hipStream_t s);
 int sl_select_tune(const char *key, int value);

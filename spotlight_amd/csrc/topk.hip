@@ -222,6 +222,13 @@ void sl_select_carve(select_args &a, void *ws, int64_t n_for_blocks) {
     a.block_cnt = reinterpret_cast<uint32_t *>(p);
     a.n_blocks = static_cast<int>((n_for_blocks + TK_BLOCK - 1) / TK_BLOCK);
     if (a.n_blocks < 1) a.n_blocks = 1;
+    a.hist_used = a.hist_groups;
+}
+
+// copies that tokens [0, n) can be counted into
+int sl_select_hist_used(const select_args &a, int64_t n) {
+    const int64_t spans = (n + a.hist_span - 1) / a.hist_span;
+    return spans < a.hist_groups ? static_cast<int>(spans < 1 ? 1 : spans) : a.hist_groups;
 }
 
 int sl_select_launch(const select_args &a, hipStream_t s) {
@@ -287,6 +294,7 @@ int topk_select_with(const int16_t *score, int64_t stride_b, int64_t stride_n, i
     a.B = B; a.KH = KH; a.k = k; a.n_bins = n_bins; a.len_bias = 0; a.n = n;
     a.stride_b = stride_b; a.stride_n = stride_n; a.stride_h = stride_h;
     sl_select_carve(a, ws, n);
+    a.hist_used = sl_select_hist_used(a, n);
     const int64_t hist_words = static_cast<int64_t>(B) * KH * n_bins * a.hist_groups;
     zero_words_kernel<<<dim3(static_cast<unsigned>((hist_words + 255) / 256)), dim3(256), 0, s>>>(a.hist, hist_words);
     if (n > 0) {

@@ -81,7 +81,7 @@ __device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, int 
         const bool live = j < BPT && bi < NB;
         const int bin = live ? NB - 1 - bi : 0;  // unconditional loads, dead bins are dropped below
 #pragma unroll
-        for (int g = 0; g < NG; ++g) raw[j][g] = gh[g * NB + bin];
+        for (int g = 0; g < NG; ++g) raw[j][g] = g < a.hist_used ? gh[g * NB + bin] : 0u;  // uniform: unused copies are skipped
     }
     uint32_t mine = 0;
 #pragma unroll
