@@ -81,6 +81,8 @@ def main():
                     help="keep the full K/V store in pinned host memory behind the LRU table (configs with LRU slots)")
     ap.add_argument("--floor-only", action="store_true",
                     help="only measure what the step's launches cost by themselves (near-empty kernels on the step's grids)")
+    ap.add_argument("--codes-layout", default="auto", choices=["auto", "token", "head"],
+                    help="key-code layout: head-major runs scorer, selection and attention as one launch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-breakdown", action="store_true")
     args = ap.parse_args()
@@ -118,7 +120,10 @@ def main():
     tokens = tokens_warm + tokens_timed + 4 + 64   # cache growth incl. the breakdown passes
     n_cap = (n0 + tokens + 7) // 8 * 8
     if args.floor_only:
-        print(json.dumps({"config": args.config, "latency_floor": latency_floor(dev, c, L, n0 + tokens, reps=64)}), flush=True)
+        blocks = (n_cap + 4095) // 4096
+        head = args.codes_layout == "head" or (args.codes_layout == "auto" and not c["lru"] and QH // KH in (1, 2, 4)
+                                               and n_cap <= 65536 and B * KH * blocks <= 256 and k <= 128 * blocks)
+        print(json.dumps({"config": args.config, "latency_floor": latency_floor(dev, c, L, n0 + tokens, reps=64, one_launch_tail=head)}), flush=True)
         return
 
     cpu_gen = torch.Generator()
@@ -143,7 +148,7 @@ def main():
             hk = hq if KH == QH else decode.HashWeights.random_linear(KH, 128, 128, dtype, dev, cpu_gen)
         st = decode.LayerDecodeState(B, QH, KH, d, n_cap, k, hq, hk, dtype=dtype, device=dev,
                                      lru_slots=c["lru"], inputs=tuple(t[0, li] for t in cur),
-                                     host_store=args.host_store)
+                                     host_store=args.host_store, codes_layout=args.codes_layout)
         # prefill in slabs to bound the transient memory of hashing
         st.seq_lens.zero_()
         slab = max(1, (1 << 22) // (B * KH))
@@ -153,7 +158,7 @@ def main():
             vv = torch.randn((B, s1 - s0, KH, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
             st.keys[:, s0:s1] = kk      # (a device-to-host copy with --host-store)
             st.vals[:, s0:s1] = vv
-            kernel.cache_append(st.codes, st.hash_k.hash_rows(kk), start=s0)
+            st.hash_k.hash_rows(kk, out=st.codes[:, s0:s1])
         st.seq_lens.fill_(n0)
         st.host_len = n0
         layers.append(st)
@@ -208,9 +213,13 @@ def main():
     if not args.no_kernel_breakdown:
         # equalise lengths (a partial token may have advanced only some layers)
         M = 4 * L
-        stage_sets = [("hash", _lib.STAGE_HASH), ("score", _lib.STAGE_SCORE),
-                      ("score+select", _lib.STAGE_SCORE | _lib.STAGE_SELECT), ("attn", _lib.STAGE_ATTN),
-                      ("select+attn", _lib.STAGE_SELECT | _lib.STAGE_ATTN)]
+        one_launch_tail = layers[0].codes_layout == "head"   # scorer + selection + attention as ONE launch
+        if one_launch_tail:
+            stage_sets = [("hash", _lib.STAGE_HASH), ("score+select+attn", _lib.STAGE_SCORE | _lib.STAGE_SELECT | _lib.STAGE_ATTN)]
+        else:
+            stage_sets = [("hash", _lib.STAGE_HASH), ("score", _lib.STAGE_SCORE),
+                          ("score+select", _lib.STAGE_SCORE | _lib.STAGE_SELECT), ("attn", _lib.STAGE_ATTN),
+                          ("select+attn", _lib.STAGE_SELECT | _lib.STAGE_ATTN)]
         if c["lru"]:
             stage_sets.insert(3, ("lru", _lib.STAGE_LRU))
         raw = {}
@@ -228,15 +237,19 @@ def main():
             torch.cuda.synchronize()
             raw[name] = e0.elapsed_time(e1) * 1e3 / M
             del g
-        raw["select"] = max(raw["score+select"] - raw["score"], 0.0)
+        if not one_launch_tail:
+            raw["select"] = max(raw["score+select"] - raw["score"], 0.0)
         ab["select+attn"] = ab["attn"]
+        ab["score+select+attn"] = ab["score"] + ab["attn"]
         # the step runs selection and attention as one launch when it can (no LRU, <= 64k rows):
         # then "select+attn" is that launch and "select" / "attn" are the two-launch alternative
         # (same rule as the library: the shape allows it and a 4096-token block keeps <= 128 rows on average)
         fused_tail = (not c["lru"] and n_cap <= 65536 and QH // KH in (1, 2, 4)
                       and k <= 128 * ((n_max + 4095) // 4096))
         names = ("hash", "score", "select+attn") if fused_tail else ("hash", "score", "select", "lru", "attn")
-        for name in ("hash", "score", "select", "lru", "attn", "select+attn"):
+        if one_launch_tail:
+            names = ("hash", "score+select+attn")
+        for name in ("hash", "score", "select", "lru", "attn", "select+attn", "score+select+attn"):
             if name in raw:
                 us = raw[name]
                 kernels[name] = {"us": round(us, 3), "algorithmic_bytes": ab[name],
@@ -254,7 +267,7 @@ def main():
                     "algorithmic_bytes_per_launch": kernels[dominant]["algorithmic_bytes"],
                     "us_per_launch": kernels[dominant]["us"]}
 
-    floor = latency_floor(dev, c, L, n_max)
+    floor = latency_floor(dev, c, L, n_max, one_launch_tail=layers[0].codes_layout == "head")
 
     cpu_baseline = cpu_reference_form = None
     if not args.no_cpu_baseline:
@@ -271,7 +284,8 @@ def main():
         "dtype": c["dtype"], "data": "synthetic",
         "config": {"workload": f"{args.config}: {c['desc']}", "batch": B, "q_heads": QH, "kv_heads": KH,
                    "head_dim": d, "context": n0, "k": k, "code_bits": 128, "hash": c["hash"],
-                   "lru_slots": c["lru"], "kv_store": "pinned host memory" if args.host_store else "hbm",
+                   "lru_slots": c["lru"], "codes_layout": layers[0].codes_layout,
+                   "launches_per_step": 2 if layers[0].codes_layout == "head" else None, "kv_store": "pinned host memory" if args.host_store else "hbm",
                    "layers_rotated": L,
                    "graph": f"one HIP graph per token ({L} steps); {tokens_timed} replays timed after {tokens_warm} warm-up replays"},
         "gpu_event_ms_per_step": round(gpu_ms / steps_timed, 6),
@@ -381,7 +395,7 @@ class E2EModel:
                         st = w["st"]
                         st.keys[b, :n0] = kk
                         st.vals[b, :n0] = vv
-                        kernel.cache_append(st.codes[b:b + 1], st.hash_k.hash_rows(kk[None]), start=0)
+                        st.hash_k.hash_rows(kk[None], out=st.codes[b:b + 1, :n0])
                     else:
                         w["kc"][b, :, :n0] = kk.transpose(0, 1)
                         w["vc"][b, :, :n0] = vv.transpose(0, 1)
@@ -501,7 +515,7 @@ def run_e2e(args):
 _STAGES_NO_ADVANCE = 1 | 2 | 4 | 16     # hash, score, select, attention launched as stages: lengths do not advance
 
 
-STAGE_KERNEL = {"hash": "hash_kernel", "score": "hamming_kernel", "select": "select_fused_kernel",
+STAGE_KERNEL = {"score+select+attn": "score_select_attend_kernel", "hash": "hash_kernel", "score": "hamming_kernel", "select": "select_fused_kernel",
                 "lru": "lru_kernel", "attn": "sparse_attn_kernel", "select+attn": "select_attend_kernel"}
 
 
@@ -525,7 +539,7 @@ def profiled_traffic(config, stage):
     return None
 
 
-def latency_floor(dev, c, L, n_max, reps=8):
+def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False):
     """What the step's launches cost by themselves on this machine: a HIP graph of L x (as many dependent
     launches as the step has, with the step's grids) of a kernel that does nothing, and of one whose lanes do a
     single dependent load.  us per step-equivalent."""
@@ -540,7 +554,9 @@ def latency_floor(dev, c, L, n_max, reps=8):
     blocks4k = (n_max + 4095) // 4096
     grids = [((QH + KH) * ((B + hash_rows - 1) // hash_rows), 512),
              (((n_max * KH + 2047) // 2048) * B, 512)]
-    if c["lru"]:
+    if one_launch_tail:
+        grids = [grids[0], (blocks4k * KH * B, 512)]
+    elif c["lru"]:
         grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
     elif QH // KH in (1, 2, 4) and n_max <= 65536 and c["k"] <= 128 * blocks4k:
         grids += [(blocks4k * KH * B, 512)]

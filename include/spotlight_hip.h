@@ -276,7 +276,11 @@ typedef struct {
     int n_layers, d_hid, residue;
     const void *w1_q, *b1_q, *w2_q, *b2_q;   /* [QH, ...]                       */
     const void *w1_k, *b1_k, *w2_k, *b2_k;   /* [KH, ...]                       */
-    /* caches, token-major */
+    /* caches, token-major; codes_head_major != 0: codes are [B, KH, n_cap, W]  */
+    /* and scorer, selection and attention run as ONE launch (needs no LRU,     */
+    /* W == 4, QH/KH in {1,2,4}, n_max <= 65536 and a grid that fits the device */
+    /* at once: otherwise SL_ERR_UNSUPPORTED, use token-major codes)            */
+    int codes_head_major;
     uint32_t *codes;        /* [B, n_cap, KH, W]                                */
     void *keys, *vals;      /* [B, n_cap, KH, d]                                */
     int32_t *seq_lens;      /* [B] tokens cached BEFORE this step; incremented  */
@@ -300,6 +304,11 @@ typedef struct {
 } sl_decode_params;
 
 size_t sl_decode_workspace_bytes(const sl_decode_params *p);
+/* Byte offset, inside the workspace, of a 32-bit word that the one-launch scorer +
+ * tail sets to 1 if a workgroup ever gave up waiting for the histograms of the other
+ * blocks of its (b, kv head) (results of that step are then wrong); (size_t)-1 when
+ * the parameters do not use that launch.  It stays 0 in a healthy run. */
+size_t sl_decode_error_offset(const sl_decode_params *p);
 int sl_decode_step(const sl_decode_params *p, void *stream);
 
 /* The same step restricted to a subset of its kernels, for profiling one

@@ -31,7 +31,7 @@ class DecodeParams(C.Structure):
         ("n_layers", c_int), ("d_hid", c_int), ("residue", c_int),
         ("w1_q", c_void_p), ("b1_q", c_void_p), ("w2_q", c_void_p), ("b2_q", c_void_p),
         ("w1_k", c_void_p), ("b1_k", c_void_p), ("w2_k", c_void_p), ("b2_k", c_void_p),
-        ("codes", c_void_p), ("keys", c_void_p), ("vals", c_void_p), ("seq_lens", c_void_p),
+        ("codes_head_major", c_int), ("codes", c_void_p), ("keys", c_void_p), ("vals", c_void_p), ("seq_lens", c_void_p),
         ("out", c_void_p), ("idx", c_void_p),
         ("lru_C", c_int), ("lru_map_cap", c_int64),
         ("slot_token", c_void_p), ("slot_stamp", c_void_p), ("token_slot", c_void_p),
@@ -64,6 +64,7 @@ SIGNATURES = {
     "sl_attn_workspace_bytes": (c_size_t, [c_int] * 5),
     "sl_sparse_gqa_attn": (c_int, [c_void_p] * 5 + [c_int] * 6 + [c_int64] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),
     "sl_decode_workspace_bytes": (c_size_t, [C.POINTER(DecodeParams)]),
+    "sl_decode_error_offset": (c_size_t, [C.POINTER(DecodeParams)]),
     "sl_decode_step": (c_int, [C.POINTER(DecodeParams), c_void_p]),
     "sl_decode_stages": (c_int, [C.POINTER(DecodeParams), c_int, c_void_p]),
     "sl_probe_launch": (c_int, [c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),

@@ -15,6 +15,7 @@
 #include <string.h>
 
 #include "attn.h"
+#include "fused_step.h"
 #include "hamming.h"
 #include "hash.h"
 #include "lru.h"
@@ -43,7 +44,7 @@ int g_fuse_select_attend = 1;  // sl_tune("fuse_select_attend", 0 | 1 | 2): neve
 // them depends on k, so they keep their place when the caller lowers or raises k on a live workspace;
 // the one k-sized region comes last.
 struct ws_layout {
-    size_t q_code, attn, n_rows, select, score, lru_fetch, total;
+    size_t q_code, attn, n_rows, fused, select, score, lru_fetch, total;
 };
 
 ws_layout layout(const sl_decode_params &p) {
@@ -54,8 +55,11 @@ ws_layout layout(const sl_decode_params &p) {
     L.q_code = off; off += sl_align_up(sizeof(uint32_t) * p.B * p.QH * W, 256);
     L.attn = off;   off += sl_align_up(sl_attn_ws_bytes(p.B, p.QH, p.KH, 1), 256);  // does not depend on k
     L.n_rows = off; off += sl_align_up(sizeof(int32_t) * p.B, 256);
-    L.select = off; off += sl_select_ws_bytes(p.B, p.KH, static_cast<int>(G * p.nbits + 1), p.n_cap);
-    L.score = off;  off += sl_align_up(sizeof(int16_t) * p.B * p.KH * static_cast<size_t>(p.n_cap), 256);
+    // head-major codes: the flags and published histograms of the one-launch scorer + tail (the flags
+    // must stay zero between calls, like the tickets); no score array, no global histogram copies
+    L.fused = off;  off += p.codes_head_major ? sl_fused_ws_bytes(p.B, p.KH) : 0;
+    L.select = off; off += p.codes_head_major ? 0 : sl_select_ws_bytes(p.B, p.KH, static_cast<int>(G * p.nbits + 1), p.n_cap);
+    L.score = off;  off += p.codes_head_major ? 0 : sl_align_up(sizeof(int16_t) * p.B * p.KH * static_cast<size_t>(p.n_cap), 256);
     L.lru_fetch = off; off += p.lru_C > 0 ? sl_align_up(sizeof(int32_t) * p.B * p.KH * static_cast<size_t>(p.k), 256) : 0;
     L.total = off;
     return L;
@@ -137,6 +141,11 @@ extern "C" size_t sl_decode_workspace_bytes(const sl_decode_params *p) {
     return layout(*p).total;
 }
 
+extern "C" size_t sl_decode_error_offset(const sl_decode_params *p) {
+    if (!p || !p->codes_head_major || p->B <= 0 || p->KH <= 0) return static_cast<size_t>(-1);
+    return layout(*p).fused + sizeof(uint32_t) * static_cast<size_t>(p->B) * p->KH * FS_MAX_PEERS;
+}
+
 extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
     return sl_decode_stages(pp, SL_STAGE_ALL, stream);
 }
@@ -176,7 +185,8 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     sk.x = p.k_new; sk.w1 = p.w1_k; sk.b1 = p.b1_k; sk.w2 = p.w2_k; sk.b2 = p.b2_k;
     sk.codes = p.codes; sk.code_row = p.seq_lens; sk.H = p.KH;
     sk.x_stride_b = static_cast<int64_t>(p.KH) * p.d;
-    sk.code_stride_b = p.n_cap * p.KH * W; sk.code_stride_h = W; sk.code_stride_n = static_cast<int64_t>(p.KH) * W;
+    if (p.codes_head_major) { sk.code_stride_b = p.n_cap * p.KH * W; sk.code_stride_h = p.n_cap * W; sk.code_stride_n = W; }
+    else { sk.code_stride_b = p.n_cap * p.KH * W; sk.code_stride_h = W; sk.code_stride_n = static_cast<int64_t>(p.KH) * W; }
     // with rotary embedding the hash launch rotates q and the new key at position seq_lens[b] first:
     // the rotated query goes to q_rot (the attention reads it from there), the rotated key into its
     // cache row (instead of the plain copy of k_new)
@@ -189,6 +199,32 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     sk.copy_src[0] = rope ? nullptr : p.k_new; sk.copy_dst[0] = p.keys;
     sk.copy_src[1] = p.v_new; sk.copy_dst[1] = p.vals;
     sk.copy_dst_stride_b = p.n_cap * p.KH * p.d; sk.copy_dst_stride_n = static_cast<int64_t>(p.KH) * p.d;
+    if (p.codes_head_major) {
+        // two launches: hash, then scorer + selection + attention over head-major codes
+        SL_REQUIRE(p.lru_C == 0 && sl_fused_step_supported(G, W, G * p.nbits + 1, p.n_max, p.B, p.KH), SL_ERR_UNSUPPORTED);
+        const int tail_stages = SL_STAGE_SCORE | SL_STAGE_SELECT | SL_STAGE_ATTN;
+        SL_REQUIRE((stages & tail_stages) == 0 || (stages & tail_stages) == tail_stages, SL_ERR_UNSUPPORTED);
+        ha.len_out = n_rows;
+        if (stages & SL_STAGE_HASH) {
+            rc = sl_hash_launch(ha, s);
+            if (rc != SL_OK) return rc;
+        }
+        if (!(stages & tail_stages)) return SL_OK;
+        fused_args fa{};
+        fa.q_code = q_code; fa.k_code = p.codes; fa.q_stride_b = static_cast<int64_t>(p.QH) * W;
+        fa.k_stride_b = p.n_cap * p.KH * W; fa.k_stride_h = p.n_cap * W; fa.head_map = p.head_map;
+        select_args fs{};
+        fs.B = p.B; fs.KH = p.KH; fs.n_bins = G * p.nbits + 1; fs.idx = p.idx; fs.seq_lens = n_rows;
+        fs.k = p.k; fs.len_bias = 0; fs.n = p.n_max;
+        attn_args fq{};
+        fq.q = p.rope_inv_freq ? p.q_rot : p.q; fq.out = p.out; fq.dtype = p.dtype; fq.B = p.B; fq.QH = p.QH; fq.KH = p.KH; fq.k = p.k;
+        fq.rows = 0; fq.scale = 0.f; fq.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
+        const bool all = stages == SL_STAGE_ALL;  // lengths only advance on a complete step
+        fq.bump_lens = all ? p.seq_lens : nullptr; fq.bump_step = all ? p.step_counter : nullptr;
+        fq.keys = p.keys; fq.vals = p.vals; fq.idx = p.idx;
+        fq.kv_stride_b = p.n_cap * p.KH * p.d; fq.kv_stride_h = p.d; fq.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
+        return sl_fused_step_launch(fa, fs, fq, ws + L.fused, ws + L.attn, attn_bytes, s);
+    }
     select_args ta{};
     ta.B = p.B; ta.KH = p.KH; ta.n_bins = G * p.nbits + 1;
     sl_select_carve(ta, ws + L.select, p.n_cap);

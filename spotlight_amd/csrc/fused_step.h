@@ -1,0 +1,23 @@
+// Scorer + count-select + sparse attention as one launch over head-major key codes.
+#pragma once
+#include "attn.h"
+#include "topk.h"
+
+constexpr int FS_MAX_PEERS = 16;   // 4096-row blocks per (b, kv head)
+constexpr int FS_NB_PAD = 1028;    // words between the published histograms of two blocks
+
+struct fused_args {
+    const uint32_t *q_code;   // [B, QH, 4], batch stride q_stride_b words
+    const uint32_t *k_code;   // head-major: word w of row t of (b, h) at b*k_stride_b + h*k_stride_h + t*4 + w
+    int64_t q_stride_b, k_stride_b, k_stride_h;
+    int head_map;
+    uint32_t *peer_hist;      // workspace (set by the launcher): [B*KH][FS_MAX_PEERS][FS_NB_PAD]
+    uint32_t *peer_flag;      // workspace: [B*KH][FS_MAX_PEERS], zero between launches
+    uint32_t *error;          // workspace: set to 1 by a workgroup that gave up waiting for a peer
+};
+
+size_t sl_fused_ws_bytes(int B, int KH);
+bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH);
+// sa: n_bins, k, idx, seq_lens (row counts), len_bias, n, B, KH; aa as for sl_attn_launch (aa.idx is ignored).
+int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, void *fused_ws, void *attn_ws, size_t attn_ws_bytes,
+                         hipStream_t s);

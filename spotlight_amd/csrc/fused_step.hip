@@ -1,0 +1,284 @@
+// Scorer + count-select + sparse attention in ONE launch: the decode step's second and last launch
+// when the key codes are stored head-major.
+//
+// With codes laid out [B, KH, n_cap, W] a workgroup can own a block of 4096 rows of ONE (b, kv head):
+// it streams the block's codes (64 KB, contiguous), keeps the 8 scores per lane in registers and
+// builds the block's score histogram in LDS.  The only thing it lacks for the selection is what the
+// other blocks of the same (b, kv head) saw, so the blocks -- at most 16, all resident at the same
+// time -- swap histograms: each publishes its 513 bins with device-coherent stores and raises a flag,
+// waits (bounded) for the flags of its peers and reads their bins.  From there on it is the fused
+// select + attend kernel: threshold from the summed histograms, kept rows in front of the block from
+// the peers with a lower block number, placement, attention over exactly its kept rows, run merge.
+// Compared with scorer launch + select/attend launch this removes a launch and the gap after it, the
+// int16 score array (written, then read back), the global histogram copies with their atomics and
+// their clearing; the swap costs about 1.2 us (measured: publish, wait for 8 peers, read 8 x 513 bins).
+//
+// Waiting on other workgroups is only safe while every workgroup of the launch can be resident at
+// once; the host checks the grid against the device's capacity for this kernel and otherwise the
+// caller must use the three-launch path (token-major codes).  The wait is bounded all the same: a
+// workgroup that gives up sets an error word and goes on, so the launch always drains.
+#include "fused_step.h"
+
+#include "attn_core.h"
+#include "topk_core.h"
+
+namespace {
+
+constexpr int FS_NW = 8;
+constexpr int FS_THREADS = FS_NW * 64;
+constexpr int FS_SLOTS = 8;                          // rows per lane: row = block*4096 + wave*512 + slot*64 + lane
+constexpr int FS_BLOCK = FS_THREADS * FS_SLOTS;      // 4096 rows
+constexpr int FS_MAX_BPT = 2;                        // histogram bins per lane (<= 1024 bins)
+constexpr uint32_t FS_SPIN_LIMIT = 1u << 22;
+
+static_assert(FS_MAX_PEERS == AT_MAX_SPLITS, "one attention run per block of rows");
+static_assert(FS_BLOCK == 4096, "block of rows");
+
+template <typename T, int G>
+__global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_args fa, select_args sa, attn_args aa) {
+    constexpr int W = 4;
+    __shared__ uint32_t s_wave[64];
+    __shared__ int s_tn[4];
+    __shared__ uint32_t s_hist[FS_THREADS * FS_MAX_BPT];
+    __shared__ uint32_t s_cnt[FS_NW];
+    __shared__ int s_range[2];
+    __shared__ int32_t s_list[FS_BLOCK];
+    __shared__ attn_shared<G, FS_NW> sh;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int bh = b * sa.KH + h;
+    const int NB = sa.n_bins;
+
+    // loads first: the G query codes of this kv head and the lane's 8 rows; none needs the row count
+    // (rows past the bound fa.n re-read the last row and are discarded below)
+    const uint32_t *qb = fa.q_code + static_cast<int64_t>(b) * fa.q_stride_b;
+    uint4 qreg[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int qh = fa.head_map == SL_HEADMAP_BLOCKED ? h * G + g : g * sa.KH + h;
+        qreg[g] = *reinterpret_cast<const uint4 *>(qb + static_cast<int64_t>(qh) * W);
+    }
+    const uint4 *kb = reinterpret_cast<const uint4 *>(fa.k_code + static_cast<int64_t>(b) * fa.k_stride_b +
+                                                      static_cast<int64_t>(h) * fa.k_stride_h);
+    const int64_t t_base = static_cast<int64_t>(blk) * FS_BLOCK + wave * (64 * FS_SLOTS) + lane;
+    uint4 kreg[FS_SLOTS];
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        const int64_t t = t_base + j * 64;
+        kreg[j] = kb[t < sa.n ? t : sa.n - 1];
+    }
+    const int64_t n_b = tokens_of(sa, b);
+    const int k_eff = n_b < sa.k ? static_cast<int>(n_b) : sa.k;
+    int32_t *out = sa.idx + static_cast<int64_t>(bh) * sa.k;
+    if (blk == 0)
+        for (int i = k_eff + tid; i < sa.k; i += FS_THREADS) out[i] = -1;
+    if (static_cast<int64_t>(blk) * FS_BLOCK >= n_b) return;
+    const int S = static_cast<int>((n_b + FS_BLOCK - 1) / FS_BLOCK);  // blocks (= attention runs) of this (b, kv head)
+
+    for (int e = tid; e < FS_THREADS * FS_MAX_BPT; e += FS_THREADS) s_hist[e] = 0;
+    if (tid == 0) { s_range[0] = NB; s_range[1] = -1; }
+    __syncthreads();
+
+    // scores: matching bits summed over the G query heads; -1 marks a row past the end
+    int sc[FS_SLOTS];
+    int s_lo = NB, s_hi = -1;
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        int dist = 0;
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+            dist += __popc(qreg[g].x ^ kreg[j].x) + __popc(qreg[g].y ^ kreg[j].y) + __popc(qreg[g].z ^ kreg[j].z) +
+                    __popc(qreg[g].w ^ kreg[j].w);
+        const bool valid = t_base + j * 64 < n_b;
+        sc[j] = valid ? G * W * 32 - dist : -1;
+        if (valid) {
+            atomicAdd(&s_hist[sc[j]], 1u);
+            s_lo = sc[j] < s_lo ? sc[j] : s_lo;
+            s_hi = sc[j] > s_hi ? sc[j] : s_hi;
+        }
+    }
+    // the block's score range: only these bins of its histogram can be non-empty
+    s_lo = wave_min_i32(s_lo);
+    s_hi = wave_max_i32(s_hi);
+    if (lane == 0) { atomicMin(&s_range[0], s_lo); atomicMax(&s_range[1], s_hi); }
+    __syncthreads();
+
+    // Histogram of the whole (b, kv head), restricted to [lo, hi], the union of the blocks' score ranges:
+    // bin hi - r is rank r.  cnt = this lane's ranks summed over the blocks, before = over the blocks in
+    // front of this one.
+    int lo = s_range[0], hi = s_range[1];   // a block that got here holds at least one row: lo <= hi
+    uint32_t cnt[FS_MAX_BPT], before[FS_MAX_BPT], mine = 0;
+    if (S > 1) {
+        uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * FS_MAX_PEERS * FS_NB_PAD;
+        uint32_t *flags = fa.peer_flag + static_cast<int64_t>(bh) * FS_MAX_PEERS;
+        // every bin is published, zeros included: the peers read the union of all ranges
+        for (int e = tid; e < NB; e += FS_THREADS) st_agent(peers + blk * FS_NB_PAD + e, s_hist[e]);
+        publish_wait();
+        __syncthreads();
+        // the flag carries the block's range: bit 31 = published, bits 12.. = hi, bits 0..11 = lo
+        if (tid == 0) st_agent(flags + blk, 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo));
+        if (wave == 0) {
+            uint32_t f = 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo);
+            if (lane < S) {
+                uint32_t spins = 0;
+                while (((f = ld_agent(flags + lane)) & 0x80000000u) == 0u) {
+                    if (++spins > FS_SPIN_LIMIT) { st_agent(fa.error, 1u); f = 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo); break; }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            const int all_lo = wave_min_i32(static_cast<int>(f & 0xfffu));
+            const int all_hi = wave_max_i32(static_cast<int>((f >> 12) & 0xfffu));
+            if (lane == 0) { s_range[0] = all_lo; s_range[1] = all_hi; }
+        }
+        __syncthreads();
+        lo = s_range[0]; hi = s_range[1];
+    }
+    const int n_ranks = hi - lo + 1;
+    const int BPT = (n_ranks + FS_THREADS - 1) / FS_THREADS;
+    if (S > 1) {
+        const uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * FS_MAX_PEERS * FS_NB_PAD;
+#pragma unroll
+        for (int j = 0; j < FS_MAX_BPT; ++j) {
+            const int r = tid * BPT + j;
+            cnt[j] = 0u; before[j] = 0u;
+            if (j < BPT && r < n_ranks) {   // the loads and their use sit in one block: one round trip for the lanes that have a rank
+                uint32_t raw[FS_MAX_PEERS];
+#pragma unroll
+                for (int g = 0; g < FS_MAX_PEERS; ++g) raw[g] = ld_agent(peers + (g < S ? g : blk) * FS_NB_PAD + (hi - r));
+                uint32_t c = 0, bf = 0;
+#pragma unroll
+                for (int g = 0; g < FS_MAX_PEERS; ++g) {
+                    const uint32_t v = g < S ? raw[g] : 0u;
+                    c += v;
+                    bf += g < blk ? v : 0u;
+                }
+                cnt[j] = c; before[j] = bf;
+            }
+            mine += cnt[j];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < FS_MAX_BPT; ++j) {
+            const int r = tid * BPT + j;
+            cnt[j] = (j < BPT && r < n_ranks) ? s_hist[hi - r] : 0u;
+            before[j] = 0u;
+            mine += cnt[j];
+        }
+    }
+
+    int thr, need;
+    uint32_t tg, te;
+    find_threshold<FS_THREADS, FS_MAX_BPT>(hi, n_ranks, cnt, before, mine, k_eff, s_wave, s_tn, thr, need, tg, te);
+
+    // placement in row order (wave, slot, lane): ballots give every kept row its position
+    uint32_t mgt_lo[FS_SLOTS], mgt_hi[FS_SLOTS], meq_lo[FS_SLOTS], meq_hi[FS_SLOTS];
+    uint32_t wave_gt = 0, wave_eq = 0;
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        const uint64_t mg = __ballot(sc[j] > thr), me = __ballot(sc[j] == thr);
+        mgt_lo[j] = static_cast<uint32_t>(mg); mgt_hi[j] = static_cast<uint32_t>(mg >> 32);
+        meq_lo[j] = static_cast<uint32_t>(me); meq_hi[j] = static_cast<uint32_t>(me >> 32);
+        wave_gt += __popc(mgt_lo[j]) + __popc(mgt_hi[j]);
+        wave_eq += __popc(meq_lo[j]) + __popc(meq_hi[j]);
+    }
+    if (lane == 0) s_cnt[wave] = wave_gt | (wave_eq << 16);
+    __syncthreads();
+    uint32_t gt_before = tg, eq_before = te, tot_gt = 0, tot_eq = 0;
+#pragma unroll
+    for (int w = 0; w < FS_NW; ++w) {
+        const uint32_t c = s_cnt[w];
+        tot_gt += c & 0xffffu; tot_eq += c >> 16;
+        gt_before += w < wave ? (c & 0xffffu) : 0u;
+        eq_before += w < wave ? (c >> 16) : 0u;
+    }
+    const uint32_t uneed = static_cast<uint32_t>(need);
+    const uint32_t first = tg + (te < uneed ? te : uneed);   // output position of the block's first kept row
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        const uint32_t g_here = gt_before + __builtin_amdgcn_mbcnt_hi(mgt_hi[j], __builtin_amdgcn_mbcnt_lo(mgt_lo[j], 0u));
+        const uint32_t e_here = eq_before + __builtin_amdgcn_mbcnt_hi(meq_hi[j], __builtin_amdgcn_mbcnt_lo(meq_lo[j], 0u));
+        const bool above = sc[j] > thr, equal = sc[j] == thr;
+        const uint32_t pos = g_here + (e_here < uneed ? e_here : uneed);
+        if ((above || (equal && e_here < uneed)) && pos < static_cast<uint32_t>(k_eff))
+            s_list[pos - first] = static_cast<int32_t>(t_base + j * 64);
+        gt_before += __popc(mgt_lo[j]) + __popc(mgt_hi[j]);
+        eq_before += __popc(meq_lo[j]) + __popc(meq_hi[j]);
+    }
+    const uint32_t eq_end = te + tot_eq;
+    uint32_t end = tg + tot_gt + (eq_end < uneed ? eq_end : uneed);
+    if (end > static_cast<uint32_t>(k_eff)) end = static_cast<uint32_t>(k_eff);
+    const int n_kept = end > first ? static_cast<int>(end - first) : 0;
+
+    // the list goes out with coalesced stores; the attention then runs over it
+    __syncthreads();
+    for (int i = tid; i < n_kept; i += FS_THREADS) out[first + i] = s_list[i];
+    attend_rows_and_merge<T, G, FS_NW>(aa, b, h, blk, S, s_list, n_kept, sh);
+}
+
+template <typename T, int G>
+int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
+    // every workgroup must be able to be resident at once: workgroups wait for their peers
+    static int slots = 0;
+    if (slots == 0) {
+        int per_cu = 0, dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G>), FS_THREADS, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            return SL_ERR_LAUNCH;
+        }
+        slots = per_cu * cus > 0 ? per_cu * cus : -1;
+    }
+    SL_REQUIRE(slots > 0 && static_cast<int64_t>(grid.x) * grid.y * grid.z <= slots, SL_ERR_UNSUPPORTED);
+    score_select_attend_kernel<T, G><<<grid, dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
+    return sl_check_launch();
+}
+
+template <typename T>
+int launch_t(const fused_args &fa, const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
+    switch (aa.QH / aa.KH) {
+        case 1: return launch_tg<T, 1>(fa, sa, aa, grid, s);
+        case 2: return launch_tg<T, 2>(fa, sa, aa, grid, s);
+        case 4: return launch_tg<T, 4>(fa, sa, aa, grid, s);
+        default: return SL_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace
+
+size_t sl_fused_ws_bytes(int B, int KH) {
+    const size_t bh = static_cast<size_t>(B) * KH;
+    return sl_align_up(sizeof(uint32_t) * (bh * FS_MAX_PEERS + 64), 256) +           // flags, then the error word
+           sl_align_up(sizeof(uint32_t) * bh * FS_MAX_PEERS * FS_NB_PAD, 256);       // published histograms
+}
+
+bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH) {
+    const int64_t blocks = (n + FS_BLOCK - 1) / FS_BLOCK;
+    return (G == 1 || G == 2 || G == 4) && W == 4 && n_bins <= FS_THREADS * FS_MAX_BPT && n_bins <= FS_NB_PAD &&
+           blocks <= FS_MAX_PEERS && B <= 65535 && KH <= 65535;
+}
+
+int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, void *fused_ws, void *attn_ws, size_t attn_ws_bytes,
+                         hipStream_t s) {
+    const int G = aa.QH / aa.KH;
+    SL_REQUIRE(sl_fused_step_supported(G, 4, sa.n_bins, sa.n, aa.B, aa.KH), SL_ERR_UNSUPPORTED);
+    SL_REQUIRE(fa.q_code && fa.k_code && fused_ws && sa.seq_lens, SL_ERR_NULL);
+    SL_REQUIRE(sl_aligned(fa.q_code, 16) && sl_aligned(fa.k_code, 16) && (fa.k_stride_b % 4) == 0 && (fa.k_stride_h % 4) == 0 &&
+               (fa.q_stride_b % 4) == 0, SL_ERR_ALIGN);
+    int rc = sl_attn_prepare(aa, attn_ws, attn_ws_bytes);
+    if (rc != SL_OK) return rc;
+    const size_t bh = static_cast<size_t>(aa.B) * aa.KH;
+    fa.peer_flag = static_cast<uint32_t *>(fused_ws);
+    fa.error = fa.peer_flag + bh * FS_MAX_PEERS;
+    fa.peer_hist = reinterpret_cast<uint32_t *>(static_cast<char *>(fused_ws) + sl_align_up(sizeof(uint32_t) * (bh * FS_MAX_PEERS + 64), 256));
+    aa.peer_flag = fa.peer_flag;
+    int64_t blocks = (sa.n + FS_BLOCK - 1) / FS_BLOCK;
+    if (blocks < 1) blocks = 1;
+    const dim3 grid(static_cast<unsigned>(blocks), aa.KH, aa.B);
+    switch (aa.dtype) {
+        case SL_F32: return launch_t<float>(fa, sa, aa, grid, s);
+        case SL_BF16: return launch_t<bf16_t>(fa, sa, aa, grid, s);
+        case SL_F16: return launch_t<f16_t>(fa, sa, aa, grid, s);
+        default: return SL_ERR_UNSUPPORTED;
+    }
+}

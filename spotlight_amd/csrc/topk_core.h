@@ -106,13 +106,14 @@ __device__ __forceinline__ uint32_t load_bins(const select_args &a, int bh, int 
 // the block (tg, te).  Both running sums come out of one scan.  s_wave: 32 words,
 // s_tn: 4 words of LDS.
 template <int NT, int MAX_BPT>
-__device__ __forceinline__ void find_threshold(const select_args &a, const uint32_t (&cnt)[MAX_BPT],
+__device__ __forceinline__ void find_threshold(int top_bin, int n_ranks, const uint32_t (&cnt)[MAX_BPT],
                                                const uint32_t (&before)[MAX_BPT], uint32_t mine, int k_eff,
                                                uint32_t *s_wave, int *s_tn, int &thr, int &need,
                                                uint32_t &tg, uint32_t &te) {
-    const int NB = a.n_bins, tid = threadIdx.x;
-    const int BPT = (NB + NT - 1) / NT;
-    if (tid == 0) { s_tn[0] = NB; s_tn[1] = 0; s_tn[2] = 0; s_tn[3] = 0; }  // selects nothing unless a lane finds the bin
+    // rank r (0 = best) is bin top_bin - r; lane tid owns the ranks tid*BPT .. tid*BPT + BPT - 1
+    const int tid = threadIdx.x;
+    const int BPT = (n_ranks + NT - 1) / NT;
+    if (tid == 0) { s_tn[0] = top_bin + 1; s_tn[1] = 0; s_tn[2] = 0; s_tn[3] = 0; }  // selects nothing unless a lane finds the bin
     uint32_t mine_before = 0;
 #pragma unroll
     for (int j = 0; j < MAX_BPT; ++j) mine_before += before[j];
@@ -121,7 +122,7 @@ __device__ __forceinline__ void find_threshold(const select_args &a, const uint3
 #pragma unroll
     for (int j = 0; j < MAX_BPT; ++j) {
         if (k_eff > 0 && cum < static_cast<uint32_t>(k_eff) && cum + cnt[j] >= static_cast<uint32_t>(k_eff)) {
-            s_tn[0] = NB - 1 - (tid * BPT + j);
+            s_tn[0] = top_bin - (tid * BPT + j);
             s_tn[1] = k_eff - static_cast<int>(cum);
             s_tn[2] = static_cast<int>(cum_before);
             s_tn[3] = static_cast<int>(before[j]);
@@ -134,6 +135,14 @@ __device__ __forceinline__ void find_threshold(const select_args &a, const uint3
     need = s_tn[1];
     tg = static_cast<uint32_t>(s_tn[2]);
     te = static_cast<uint32_t>(s_tn[3]);
+}
+
+template <int NT, int MAX_BPT>
+__device__ __forceinline__ void find_threshold(const select_args &a, const uint32_t (&cnt)[MAX_BPT],
+                                               const uint32_t (&before)[MAX_BPT], uint32_t mine, int k_eff,
+                                               uint32_t *s_wave, int *s_tn, int &thr, int &need,
+                                               uint32_t &tg, uint32_t &te) {
+    find_threshold<NT, MAX_BPT>(a.n_bins - 1, a.n_bins, cnt, before, mine, k_eff, s_wave, s_tn, thr, need, tg, te);
 }
 
 __device__ __forceinline__ uint32_t count_run(const uint4 &r, int thr) {

@@ -77,7 +77,8 @@ class LayerDecodeState:
     def __init__(self, batch_size: int, num_heads: int, num_kv_heads: int, head_dim: int, n_cap: int, k: int,
                  hash_q: HashWeights, hash_k: HashWeights, dtype=torch.bfloat16, device="cuda",
                  head_map: str = "blocked", lru_slots: int = 0, inputs=None, host_store: bool = False,
-                 rope_theta: Optional[float] = None, rope_inv_freq: Optional[torch.Tensor] = None):
+                 rope_theta: Optional[float] = None, rope_inv_freq: Optional[torch.Tensor] = None,
+                 codes_layout: str = "auto"):
         assert head_dim == 128, "the attention kernel covers head_dim 128"
         assert n_cap % 8 == 0, "n_cap must be a multiple of 8"
         assert hash_q.nbits == hash_k.nbits and hash_q.n_layers == hash_k.n_layers
@@ -90,7 +91,23 @@ class LayerDecodeState:
         self.head_map = head_map
         dev = self.device
         B, QH, KH, d, W = self.B, self.QH, self.KH, self.d, self.W
-        self.codes = torch.zeros((B, n_cap, KH, W), dtype=torch.uint32, device=dev)
+        # Key codes: token-major [B, n_cap, KH, W] (the reference's layout, attn_k4_q28.cu:55) for the
+        # three-launch step, or head-major [B, KH, n_cap, W] for the step whose scorer, selection and
+        # attention are ONE launch (a workgroup then owns 4096 contiguous rows of one kv head).  "auto"
+        # takes head-major whenever that launch covers the shape.  ``codes`` is always indexed
+        # [b, row, kv head, word]; with head-major storage it is a strided view.
+        if codes_layout == "auto":
+            blocks = (n_cap + 4095) // 4096
+            codes_layout = "head" if (not lru_slots and QH // KH in (1, 2, 4) and W == 4 and n_cap <= 65536
+                                      and B * KH * blocks <= 256 and k <= 128 * blocks) else "token"
+        assert codes_layout in ("token", "head")
+        self.codes_layout = codes_layout
+        if codes_layout == "head":
+            self._codes = torch.zeros((B, KH, n_cap, W), dtype=torch.uint32, device=dev)
+            self.codes = self._codes.permute(0, 2, 1, 3)
+        else:
+            self._codes = torch.zeros((B, n_cap, KH, W), dtype=torch.uint32, device=dev)
+            self.codes = self._codes
         # host_store: the full K / V store lives in pinned host memory, which the step's
         # kernels append to and fetch missed rows from in place; the GPU then only
         # holds the codes and the LRU resident table the attention reads
@@ -160,7 +177,8 @@ class LayerDecodeState:
         ptr = lambda t: t.data_ptr() if t is not None else None
         p.w1_q, p.b1_q, p.w2_q, p.b2_q = ptr(hq.w1), ptr(hq.b1), ptr(hq.w2), ptr(hq.b2)
         p.w1_k, p.b1_k, p.w2_k, p.b2_k = ptr(hk.w1), ptr(hk.b1), ptr(hk.w2), ptr(hk.b2)
-        p.codes, p.keys, p.vals = self.codes.data_ptr(), K.device_ptr(self.keys), K.device_ptr(self.vals)
+        p.codes_head_major = int(self.codes_layout == "head")
+        p.codes, p.keys, p.vals = self._codes.data_ptr(), K.device_ptr(self.keys), K.device_ptr(self.vals)
         p.seq_lens, p.out, p.idx = self.seq_lens.data_ptr(), self.out.data_ptr(), self.idx.data_ptr()
         p.step_counter = self.step_counter.data_ptr()
         p.lru_C = self.lru_slots
@@ -178,11 +196,7 @@ class LayerDecodeState:
         [B,n0,KH,W] are hashed from the keys when not given."""
         n0 = keys.shape[1]
         assert self.host_len == 0 and n0 < self.n_cap
-        if codes is None:
-            codes = self.hash_k.hash_rows(keys)
-        K.cache_append(self.keys, keys.contiguous())
-        K.cache_append(self.vals, vals.contiguous())
-        K.cache_append(self.codes, codes.contiguous())
+        self.load_rows(keys, vals, 0, codes)
         self.seq_lens.fill_(n0)
         self.host_len = n0
 
@@ -192,11 +206,13 @@ class LayerDecodeState:
         afterwards with ``set_length``.  Bounds the transient memory of hashing."""
         t = keys.shape[1]
         assert start + t < self.n_cap
-        if codes is None:
-            codes = self.hash_k.hash_rows(keys)
         K.cache_append(self.keys, keys.contiguous(), start=start)
         K.cache_append(self.vals, vals.contiguous(), start=start)
-        K.cache_append(self.codes, codes.contiguous(), start=start)
+        dst = self.codes[:, start:start + t]
+        if codes is None:
+            self.hash_k.hash_rows(keys.contiguous(), out=dst)      # hashed straight into the cache, whatever its layout
+        else:
+            dst.view(torch.int32).copy_(codes.view(torch.int32))
 
     def set_length(self, n: int) -> None:
         assert 0 <= n < self.n_cap
@@ -223,6 +239,14 @@ class LayerDecodeState:
         with torch.cuda.device(self.device):
             _lib.check(_L.sl_workspace_init(self.ws.data_ptr(), self.ws.numel(),
                                             torch.cuda.current_stream().cuda_stream), "sl_workspace_init")
+
+    def peer_wait_failed(self) -> bool:
+        """True if a workgroup of the one-launch scorer + tail ever gave up waiting for its peers (one
+        device read; always False with token-major codes)."""
+        off = _L.sl_decode_error_offset(C.byref(self.params))
+        if off == C.c_size_t(-1).value:
+            return False
+        return bool(self.ws[off:off + 4].view(torch.int32).item())
 
     def set_k(self, k: int) -> None:
         """Tokens kept per (b, kv head) from the next step on (at most the k given at

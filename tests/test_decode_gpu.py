@@ -26,7 +26,8 @@ def _gen(seed):
     return g
 
 
-def _make_state(decode, g, B, QH, KH, n0, n_cap, k, dtype, kind="mlp", lru=0, scale=0.05, head_map="blocked"):
+def _make_state(decode, g, B, QH, KH, n0, n_cap, k, dtype, kind="mlp", lru=0, scale=0.05, head_map="blocked",
+                codes_layout="auto"):
     if kind == "mlp":
         hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, DEV, g, scale=scale)
         hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, DEV, g, scale=scale)
@@ -34,7 +35,7 @@ def _make_state(decode, g, B, QH, KH, n0, n_cap, k, dtype, kind="mlp", lru=0, sc
         hq = decode.HashWeights.random_linear(QH, 128, 128, dtype, DEV, g)
         hk = hq if KH == QH else decode.HashWeights.random_linear(KH, 128, 128, dtype, DEV, g)
     st = decode.LayerDecodeState(B, QH, KH, 128, n_cap, k, hq, hk, dtype=dtype, device=DEV,
-                                 head_map=head_map, lru_slots=lru)
+                                 head_map=head_map, lru_slots=lru, codes_layout=codes_layout)
     keys = torch.randn(B, n0, KH, 128, generator=g).to(dtype)
     vals = torch.randn(B, n0, KH, 128, generator=g).to(dtype)
     st.prefill(keys.to(DEV), vals.to(DEV))
@@ -68,6 +69,7 @@ def _check_step(kernel, st, q, k_new, v_new, out, n_before, dtype):
     want = orc.sparse_attention(q.float().numpy(), keys, vals, want_idx)
     err = np.abs(out.float().cpu().numpy() - want).max()
     assert err <= TOL[dtype], err
+    assert not st.peer_wait_failed()
 
 
 DECODE_CASES = [
@@ -81,11 +83,12 @@ DECODE_CASES = [
 ]
 
 
+@pytest.mark.parametrize("layout", ["auto", "token"])
 @pytest.mark.parametrize("B,QH,KH,n0,k,dtype,kind", DECODE_CASES)
-def test_decode_step_matches_oracle(env, B, QH, KH, n0, k, dtype, kind):
+def test_decode_step_matches_oracle(env, B, QH, KH, n0, k, dtype, kind, layout):
     decode, kernel = env
     g = _gen(n0 + k)
-    st = _make_state(decode, g, B, QH, KH, n0, 2048 + 64, k, dtype, kind)
+    st = _make_state(decode, g, B, QH, KH, n0, 2048 + 64, k, dtype, kind, codes_layout=layout)
     for step in range(3):
         q = torch.randn(B, QH, 128, generator=g).to(dtype)
         k_new = torch.randn(B, KH, 128, generator=g).to(dtype)
@@ -259,7 +262,7 @@ def test_decode_with_lru_gives_identical_attention(env, fuse):
     dtype = torch.bfloat16
     _lib.check(L.sl_tune(b"fuse_select_attend", fuse), "sl_tune")
     try:
-        plain = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype)
+        plain = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype, codes_layout="token")
         lru = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype, lru=64)
         models = [[orc.LruModel(64) for _ in range(8)] for _ in range(2)]
         g = _gen(61)
@@ -300,7 +303,7 @@ def test_decode_step_two_launch_tail_matches_oracle(env, B, QH, KH, n0, k, dtype
     _lib.check(L.sl_tune(b"fuse_select_attend", 0), "sl_tune")
     try:
         g = _gen(n0 + k + 1)
-        st = _make_state(decode, g, B, QH, KH, n0, 2048 + 64, k, dtype, kind)
+        st = _make_state(decode, g, B, QH, KH, n0, 2048 + 64, k, dtype, kind, codes_layout="token")
         for step in range(2):
             q = torch.randn(B, QH, 128, generator=g).to(dtype)
             k_new = torch.randn(B, KH, 128, generator=g).to(dtype)
@@ -317,9 +320,11 @@ def test_decode_many_blocks_and_long_cache(env):
     spans with 16 and with 32 histogram copies (single-launch selection); and the
     two-launch selector once the copies wrap around (beyond 256k tokens)."""
     decode, kernel = env
-    for n0, k in ((9000, 180), (20000, 100), (70000, 300), (140000, 500), (270000, 64)):
+    for n0, k, layout in ((9000, 180, "token"), (9000, 180, "head"), (20000, 100, "token"), (20000, 100, "head"),
+                          (60000, 300, "head"), (70000, 300, "auto"), (140000, 500, "auto"), (270000, 64, "auto")):
         g = _gen(n0)
-        st = _make_state(decode, g, 1, 8, 2, n0, (n0 + 64 + 7) // 8 * 8, k, torch.bfloat16)
+        st = _make_state(decode, g, 1, 8, 2, n0, (n0 + 64 + 7) // 8 * 8, k, torch.bfloat16, codes_layout=layout)
+        assert st.codes_layout == ("token" if n0 > 65000 else layout if layout != "auto" else "head")
         for step in range(2):
             q = torch.randn(1, 8, 128, generator=g).to(torch.bfloat16)
             kn = torch.randn(1, 2, 128, generator=g).to(torch.bfloat16)
@@ -348,13 +353,14 @@ def _random_cases(count, seed):
     return cases
 
 
+@pytest.mark.parametrize("layout", ["auto", "token"])
 @pytest.mark.parametrize("B,QH,KH,n0,k,dtype,kind", _random_cases(24, 2024))
-def test_decode_step_random_shapes(env, B, QH, KH, n0, k, dtype, kind):
+def test_decode_step_random_shapes(env, B, QH, KH, n0, k, dtype, kind, layout):
     """Seeded sweep over head counts, group sizes, batch sizes, cache lengths around the
     block / tile / span boundaries, budgets above and below the cache length."""
     decode, kernel = env
     g = _gen(QH * 131 + n0 + k)
-    st = _make_state(decode, g, B, QH, KH, n0, (n0 + 16 + 7) // 8 * 8, k, dtype, kind)
+    st = _make_state(decode, g, B, QH, KH, n0, (n0 + 16 + 7) // 8 * 8, k, dtype, kind, codes_layout=layout)
     for step in range(2):
         q = torch.randn(B, QH, 128, generator=g).to(dtype)
         k_new = torch.randn(B, KH, 128, generator=g).to(dtype)

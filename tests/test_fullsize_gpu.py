@@ -104,9 +104,10 @@ def check_step_properties(st, q, kn, vn, out, n):
         assert int(st.token_slot[:, :, n - 1].min()) >= 0
 
 
-def _prefilled(decode, B, QH, KH, n0, k, dtype, kind, lru, g, cg, n_cap=None):
+def _prefilled(decode, B, QH, KH, n0, k, dtype, kind, lru, g, cg, n_cap=None, layout="auto"):
     hq, hk = _weights(decode, kind, QH, KH, dtype, cg)
-    st = decode.LayerDecodeState(B, QH, KH, 128, n_cap or (n0 + 64 + 7) // 8 * 8, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru)
+    st = decode.LayerDecodeState(B, QH, KH, 128, n_cap or (n0 + 64 + 7) // 8 * 8, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru,
+                                 codes_layout=layout)
     slab = max(1, (1 << 21) // (B * KH))   # bounds the transient memory of hashing the rows
     for s0 in range(0, n0, slab):
         s1 = min(n0, s0 + slab)
@@ -121,12 +122,13 @@ def _fresh(g, B, QH, KH, dtype):
     return tuple(torch.randn((B, h, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype) for h in (QH, KH, KH))
 
 
-@pytest.mark.parametrize("name", list(SHAPES))
+@pytest.mark.parametrize("name,layout", [(n, "auto") for n in SHAPES] + [("c2", "token")])
 @torch.no_grad()
-def test_full_size_step_properties(decode, name):
+def test_full_size_step_properties(decode, name, layout):
     B, QH, KH, n0, k, dtype, kind, lru = SHAPES[name]
     g = torch.Generator(device=DEV).manual_seed(7)
-    st = _prefilled(decode, B, QH, KH, n0, k, dtype, kind, lru, g, torch.Generator().manual_seed(7))
+    st = _prefilled(decode, B, QH, KH, n0, k, dtype, kind, lru, g, torch.Generator().manual_seed(7), layout=layout)
+    assert st.codes_layout == ("head" if name == "c2" and layout == "auto" else "token")
     for step in range(2):
         q, kn, vn = _fresh(g, B, QH, KH, dtype)
         out = st.step(q, kn, vn).clone()
@@ -142,7 +144,7 @@ def test_fused_tail_large_batch_across_block_boundary(decode):
     B, QH, KH, k, dtype = 32, 32, 8, 655, torch.bfloat16
     n0 = 8 * 4096 - 1
     g = torch.Generator(device=DEV).manual_seed(11)
-    st = _prefilled(decode, B, QH, KH, n0, k, dtype, "mlp", 0, g, torch.Generator().manual_seed(11))
+    st = _prefilled(decode, B, QH, KH, n0, k, dtype, "mlp", 0, g, torch.Generator().manual_seed(11), layout="token")
     n = n0
     for step in range(2):
         q, kn, vn = _fresh(g, B, QH, KH, dtype)

@@ -31,8 +31,10 @@ def _pair(env, B, QH, KH, n0, k, lru, seed):
     inputs = tuple(torch.zeros((B, h, 128), dtype=dtype, device=DEV) for h in (QH, KH, KH))
     n_cap = (n0 + REPLAYS + 72) // 8 * 8
     g = torch.Generator(device=DEV).manual_seed(seed)
-    states = [decode.LayerDecodeState(B, QH, KH, 128, n_cap, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru, inputs=inputs)
-              for _ in range(2)]
+    # `multi` takes the layout the step picks by itself (head-major at the headline shape: scorer, selection and
+    # attention in one launch, blocks swapping histograms); `single` is the three-launch step on token-major codes
+    states = [decode.LayerDecodeState(B, QH, KH, 128, n_cap, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru, inputs=inputs,
+                                      codes_layout=layout) for layout in ("auto", "token")]
     slab = max(1, (1 << 21) // (B * KH))
     for s0 in range(0, n0, slab):
         s1 = min(n0, s0 + slab)
