@@ -146,6 +146,12 @@ extern "C" size_t sl_decode_error_offset(const sl_decode_params *p) {
     return layout(*p).fused + sizeof(uint32_t) * static_cast<size_t>(p->B) * p->KH * FS_MAX_PEERS;
 }
 
+extern "C" int sl_decode_head_major_blocks(int dtype, int QH, int KH) {
+    SL_REQUIRE(QH > 0 && KH > 0 && QH % KH == 0, SL_ERR_SHAPE);
+    const int slots = sl_fused_step_slots(dtype, QH / KH);
+    return slots > 0 ? slots : 0;
+}
+
 extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
     return sl_decode_stages(pp, SL_STAGE_ALL, stream);
 }

@@ -18,6 +18,8 @@ struct fused_args {
 
 size_t sl_fused_ws_bytes(int B, int KH);
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH);
+// workgroups of the launch the current device holds at once (its grid may not be larger); <= 0: unknown / no such flavour
+int sl_fused_step_slots(int dtype, int G);
 // sa: n_bins, k, idx, seq_lens (row counts), len_bias, n, B, KH; aa as for sl_attn_launch (aa.idx is ignored).
 int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, void *fused_ws, void *attn_ws, size_t attn_ws_bytes,
                          hipStream_t s);

@@ -216,19 +216,37 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     attend_rows_and_merge<T, G, FS_NW>(aa, b, h, blk, S, s_list, n_kept, sh);
 }
 
+// workgroups of the kernel the device holds at once (looked up once per flavour), <= 0 when unknown
 template <typename T, int G>
-int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
-    // every workgroup must be able to be resident at once: workgroups wait for their peers
+int slots_tg() {
     static int slots = 0;
     if (slots == 0) {
         int per_cu = 0, dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
             hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G>), FS_THREADS, 0) != hipSuccess) {
             (void)hipGetLastError();
-            return SL_ERR_LAUNCH;
+            return 0;
         }
         slots = per_cu * cus > 0 ? per_cu * cus : -1;
     }
+    return slots;
+}
+
+template <typename T>
+int slots_t(int G) {
+    switch (G) {
+        case 1: return slots_tg<T, 1>();
+        case 2: return slots_tg<T, 2>();
+        case 4: return slots_tg<T, 4>();
+        default: return -1;
+    }
+}
+
+template <typename T, int G>
+int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
+    // every workgroup must be able to be resident at once: workgroups wait for their peers
+    const int slots = slots_tg<T, G>();
+    if (slots == 0) return SL_ERR_LAUNCH;
     SL_REQUIRE(slots > 0 && static_cast<int64_t>(grid.x) * grid.y * grid.z <= slots, SL_ERR_UNSUPPORTED);
     score_select_attend_kernel<T, G><<<grid, dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
     return sl_check_launch();
@@ -250,6 +268,15 @@ size_t sl_fused_ws_bytes(int B, int KH) {
     const size_t bh = static_cast<size_t>(B) * KH;
     return sl_align_up(sizeof(uint32_t) * (bh * FS_MAX_PEERS + 64), 256) +           // flags, then the error word
            sl_align_up(sizeof(uint32_t) * bh * FS_MAX_PEERS * FS_NB_PAD, 256);       // published histograms
+}
+
+int sl_fused_step_slots(int dtype, int G) {
+    switch (dtype) {
+        case SL_F32: return slots_t<float>(G);
+        case SL_BF16: return slots_t<bf16_t>(G);
+        case SL_F16: return slots_t<f16_t>(G);
+        default: return -1;
+    }
 }
 
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH) {

@@ -98,8 +98,12 @@ class LayerDecodeState:
         # [b, row, kv head, word]; with head-major storage it is a strided view.
         if codes_layout == "auto":
             blocks = (n_cap + 4095) // 4096
-            codes_layout = "head" if (not lru_slots and QH // KH in (1, 2, 4) and W == 4 and n_cap <= 65536
-                                      and B * KH * blocks <= 256 and k <= 128 * blocks) else "token"
+            fits = 0
+            if not lru_slots and QH // KH in (1, 2, 4) and W == 4 and n_cap <= 65536 and k <= 128 * blocks:
+                # all blocks of a launch must be resident at once; the library knows how many the device holds
+                with torch.cuda.device(dev):
+                    fits = _lib.load().sl_decode_head_major_blocks(K._DTYPES[self.dtype], QH, KH)
+            codes_layout = "head" if B * KH * blocks <= fits else "token"
         assert codes_layout in ("token", "head")
         self.codes_layout = codes_layout
         if codes_layout == "head":
