@@ -214,14 +214,16 @@ def main():
         # equalise lengths (a partial token may have advanced only some layers)
         M = 4 * L
         one_launch_tail = layers[0].codes_layout == "head"   # scorer + selection + attention as ONE launch
-        if one_launch_tail:
+        if one_launch_tail and c["lru"]:    # the launch ends at the selection: table update and attention follow
+            stage_sets = [("hash", _lib.STAGE_HASH), ("score+select", _lib.STAGE_SCORE | _lib.STAGE_SELECT), ("attn", _lib.STAGE_ATTN)]
+        elif one_launch_tail:
             stage_sets = [("hash", _lib.STAGE_HASH), ("score+select+attn", _lib.STAGE_SCORE | _lib.STAGE_SELECT | _lib.STAGE_ATTN)]
         else:
             stage_sets = [("hash", _lib.STAGE_HASH), ("score", _lib.STAGE_SCORE),
                           ("score+select", _lib.STAGE_SCORE | _lib.STAGE_SELECT), ("attn", _lib.STAGE_ATTN),
                           ("select+attn", _lib.STAGE_SELECT | _lib.STAGE_ATTN)]
         if c["lru"]:
-            stage_sets.insert(3, ("lru", _lib.STAGE_LRU))
+            stage_sets.insert(2 if one_launch_tail else 3, ("lru", _lib.STAGE_LRU))
         raw = {}
         for name, mask in stage_sets:
             def body(mask=mask):
@@ -241,6 +243,7 @@ def main():
             raw["select"] = max(raw["score+select"] - raw["score"], 0.0)
         ab["select+attn"] = ab["attn"]
         ab["score+select+attn"] = ab["score"] + ab["attn"]
+        ab["score+select"] = ab["score"]
         # the step runs selection and attention as one launch when it can (no LRU, <= 64k rows):
         # then "select+attn" is that launch and "select" / "attn" are the two-launch alternative
         # (same rule as the library: the shape allows it and a 4096-token block keeps <= 128 rows on average)
@@ -248,8 +251,10 @@ def main():
                       and k <= 128 * ((n_max + 4095) // 4096))
         names = ("hash", "score", "select+attn") if fused_tail else ("hash", "score", "select", "lru", "attn")
         if one_launch_tail:
-            names = ("hash", "score+select+attn")
-        for name in ("hash", "score", "select", "lru", "attn", "select+attn", "score+select+attn"):
+            names = ("hash", "score+select", "lru", "attn") if c["lru"] else ("hash", "score+select+attn")
+        for name in ("hash", "score", "select", "score+select", "lru", "attn", "select+attn", "score+select+attn"):
+            if name == "score+select" and not (one_launch_tail and c["lru"]):
+                continue
             if name in raw:
                 us = raw[name]
                 kernels[name] = {"us": round(us, 3), "algorithmic_bytes": ab[name],
@@ -285,7 +290,7 @@ def main():
         "config": {"workload": f"{args.config}: {c['desc']}", "batch": B, "q_heads": QH, "kv_heads": KH,
                    "head_dim": d, "context": n0, "k": k, "code_bits": 128, "hash": c["hash"],
                    "lru_slots": c["lru"], "codes_layout": layers[0].codes_layout,
-                   "launches_per_step": 2 if layers[0].codes_layout == "head" else None, "kv_store": "pinned host memory" if args.host_store else "hbm",
+                   "launches_per_step": floor["launches_per_step"] if floor else None, "kv_store": "pinned host memory" if args.host_store else "hbm",
                    "layers_rotated": L,
                    "graph": f"one HIP graph per token ({L} steps); {tokens_timed} replays timed after {tokens_warm} warm-up replays"},
         "gpu_event_ms_per_step": round(gpu_ms / steps_timed, 6),
@@ -515,7 +520,7 @@ def run_e2e(args):
 _STAGES_NO_ADVANCE = 1 | 2 | 4 | 16     # hash, score, select, attention launched as stages: lengths do not advance
 
 
-STAGE_KERNEL = {"score+select+attn": "score_select_attend_kernel", "hash": "hash_kernel", "score": "hamming_kernel", "select": "select_fused_kernel",
+STAGE_KERNEL = {"score+select+attn": "score_select_attend_kernel", "score+select": "score_select_attend_kernel", "hash": "hash_kernel", "score": "hamming_kernel", "select": "select_fused_kernel",
                 "lru": "lru_kernel", "attn": "sparse_attn_kernel", "select+attn": "select_attend_kernel"}
 
 
@@ -555,7 +560,11 @@ def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False):
     grids = [((QH + KH) * ((B + hash_rows - 1) // hash_rows), 512),
              (((n_max * KH + 2047) // 2048) * B, 512)]
     if one_launch_tail:
-        grids = [grids[0], (blocks4k * KH * B, 512)]
+        # blocks of 4096 rows while the device holds them all at once (two 8-wave workgroups per compute unit), else 8192
+        blocks = blocks4k if blocks4k * KH * B <= 512 else (n_max + 8191) // 8192
+        grids = [grids[0], (blocks * KH * B, 512)]
+        if c["lru"]:
+            grids += [(B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
     elif c["lru"]:
         grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
     elif QH // KH in (1, 2, 4) and n_max <= 65536 and c["k"] <= 128 * blocks4k:

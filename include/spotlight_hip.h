@@ -309,13 +309,13 @@ size_t sl_decode_workspace_bytes(const sl_decode_params *p);
  * blocks of its (b, kv head) (results of that step are then wrong); (size_t)-1 when
  * the parameters do not use that launch.  It stays 0 in a healthy run. */
 size_t sl_decode_error_offset(const sl_decode_params *p);
-/* How many 4096-row blocks, summed over all (b, kv head), a step over head-major codes
- * can take on the current device: B * KH * ceil(n_max / 4096) may not exceed it (the
- * blocks of a launch wait for each other, so all of them must be resident at once;
- * beyond it sl_decode_step returns SL_ERR_UNSUPPORTED and the caller keeps token-major
- * codes).  0 when this dtype / QH / KH has no head-major flavour; negative on bad
- * arguments.  No counterpart in the reference. */
-int sl_decode_head_major_blocks(int dtype, int QH, int KH);
+/* 1 if sl_decode_step can run this shape over head-major codes on the current
+ * device, 0 if not (the caller then keeps token-major codes), negative on bad
+ * arguments.  The blocks of rows of such a launch (4096 rows, or 8192 when that is
+ * what fits) wait for each other, so B * KH * blocks may not exceed the workgroups
+ * the device holds at once; n_max is the largest row bound the caller will pass
+ * (its n_cap).  No counterpart in the reference. */
+int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int with_lru);
 int sl_decode_step(const sl_decode_params *p, void *stream);
 
 /* The same step restricted to a subset of its kernels, for profiling one

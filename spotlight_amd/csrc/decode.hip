@@ -3,6 +3,7 @@
 // sl_decode_step enqueues, on one stream and without host synchronisation:
 //   1. hash_kernel       q codes -> workspace; new key's code, K and V -> cache row seq_lens[b];
 //                        clears the score histogram
+//   (head-major key codes: 2 + 3 (+ 5 without an LRU table) are one launch, score_select_attend_kernel)
 //   2. hamming_kernel    fused flavour: head-major scores + global histogram over seq_lens[b]+1 rows
 //   3. select_fused_kernel (or select_count_kernel + select_compact_kernel beyond 64k rows)
 //                        threshold from the histogram, stable compaction -> idx
@@ -101,7 +102,7 @@ extern "C" int sl_version(void) { return 100; }
 extern "C" int sl_tune(const char *key, int value) {
     SL_REQUIRE(key, SL_ERR_NULL);
     if (!strcmp(key, "fuse_select_attend") && value >= 0 && value <= 2) { g_fuse_select_attend = value; return SL_OK; }
-    if (sl_attn_tune(key, value) == SL_OK || sl_select_tune(key, value) == SL_OK) return SL_OK;
+    if (sl_attn_tune(key, value) == SL_OK || sl_select_tune(key, value) == SL_OK || sl_fused_tune(key, value) == SL_OK) return SL_OK;
     return sl_hash_tune(key, value);
 }
 
@@ -146,10 +147,14 @@ extern "C" size_t sl_decode_error_offset(const sl_decode_params *p) {
     return layout(*p).fused + sizeof(uint32_t) * static_cast<size_t>(p->B) * p->KH * FS_MAX_PEERS;
 }
 
-extern "C" int sl_decode_head_major_blocks(int dtype, int QH, int KH) {
-    SL_REQUIRE(QH > 0 && KH > 0 && QH % KH == 0, SL_ERR_SHAPE);
-    const int slots = sl_fused_step_slots(dtype, QH / KH);
-    return slots > 0 ? slots : 0;
+extern "C" int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int with_lru) {
+    SL_REQUIRE(B > 0 && QH > 0 && KH > 0 && QH % KH == 0 && nbits > 0 && nbits % 32 == 0 && n_max > 0, SL_ERR_SHAPE);
+    const int G = QH / KH;
+    if (!sl_fused_step_supported(G, nbits / 32, G * nbits + 1, n_max, B, KH)) return 0;
+    const int64_t heads = static_cast<int64_t>(B) * KH;
+    const int64_t b8 = (n_max + 4095) / 4096, b16 = (n_max + 8191) / 8192;
+    if (b8 <= FS_MAX_PEERS && heads * b8 <= sl_fused_step_slots(dtype, G, 4096, !with_lru)) return 1;
+    return b16 <= FS_MAX_PEERS && heads * b16 <= sl_fused_step_slots(dtype, G, 8192, !with_lru) ? 1 : 0;
 }
 
 extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
@@ -205,62 +210,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     sk.copy_src[0] = rope ? nullptr : p.k_new; sk.copy_dst[0] = p.keys;
     sk.copy_src[1] = p.v_new; sk.copy_dst[1] = p.vals;
     sk.copy_dst_stride_b = p.n_cap * p.KH * p.d; sk.copy_dst_stride_n = static_cast<int64_t>(p.KH) * p.d;
-    if (p.codes_head_major) {
-        // two launches: hash, then scorer + selection + attention over head-major codes
-        SL_REQUIRE(p.lru_C == 0 && sl_fused_step_supported(G, W, G * p.nbits + 1, p.n_max, p.B, p.KH), SL_ERR_UNSUPPORTED);
-        const int tail_stages = SL_STAGE_SCORE | SL_STAGE_SELECT | SL_STAGE_ATTN;
-        SL_REQUIRE((stages & tail_stages) == 0 || (stages & tail_stages) == tail_stages, SL_ERR_UNSUPPORTED);
-        ha.len_out = n_rows;
-        if (stages & SL_STAGE_HASH) {
-            rc = sl_hash_launch(ha, s);
-            if (rc != SL_OK) return rc;
-        }
-        if (!(stages & tail_stages)) return SL_OK;
-        fused_args fa{};
-        fa.q_code = q_code; fa.k_code = p.codes; fa.q_stride_b = static_cast<int64_t>(p.QH) * W;
-        fa.k_stride_b = p.n_cap * p.KH * W; fa.k_stride_h = p.n_cap * W; fa.head_map = p.head_map;
-        select_args fs{};
-        fs.B = p.B; fs.KH = p.KH; fs.n_bins = G * p.nbits + 1; fs.idx = p.idx; fs.seq_lens = n_rows;
-        fs.k = p.k; fs.len_bias = 0; fs.n = p.n_max;
-        attn_args fq{};
-        fq.q = p.rope_inv_freq ? p.q_rot : p.q; fq.out = p.out; fq.dtype = p.dtype; fq.B = p.B; fq.QH = p.QH; fq.KH = p.KH; fq.k = p.k;
-        fq.rows = 0; fq.scale = 0.f; fq.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
-        const bool all = stages == SL_STAGE_ALL;  // lengths only advance on a complete step
-        fq.bump_lens = all ? p.seq_lens : nullptr; fq.bump_step = all ? p.step_counter : nullptr;
-        fq.keys = p.keys; fq.vals = p.vals; fq.idx = p.idx;
-        fq.kv_stride_b = p.n_cap * p.KH * p.d; fq.kv_stride_h = p.d; fq.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
-        return sl_fused_step_launch(fa, fs, fq, ws + L.fused, ws + L.attn, attn_bytes, s);
-    }
-    select_args ta{};
-    ta.B = p.B; ta.KH = p.KH; ta.n_bins = G * p.nbits + 1;
-    sl_select_carve(ta, ws + L.select, p.n_cap);
-    ta.hist_used = sl_select_hist_used(ta, p.n_max);
-    // the scorer of this step starts from a clean histogram: per (b, kv head) the copies this launch can reach
-    ha.zero_words = ta.hist;
-    ha.zero_rows = p.B * p.KH;
-    ha.zero_count = static_cast<int64_t>(ta.n_bins) * ta.hist_used;
-    ha.zero_stride = static_cast<int64_t>(ta.n_bins) * ta.hist_groups;
-    ha.len_out = n_rows;
-    // 2. score seq_lens[b] + 1 rows
-    hamming_args sa{};
-    sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.hist_span = ta.hist_span; sa.seq_lens = n_rows;
-    sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
-    sa.n_bins = G * p.nbits + 1; sa.len_bias = 0; sa.n = p.n_max; sa.n_cap = p.n_cap;
-    sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
-    if (stages & SL_STAGE_HASH) {
-        rc = sl_hash_launch(ha, s);
-        if (rc != SL_OK) return rc;
-    }
-    if (stages & SL_STAGE_SCORE) {
-        rc = sl_hamming_launch(sa, true, s);
-        if (rc != SL_OK) return rc;
-    }
-
-    // 3. select
-    ta.score = score; ta.idx = p.idx; ta.seq_lens = n_rows;
-    ta.k = p.k; ta.len_bias = 0; ta.n = p.n_max;
-    ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
-    // 3. select -- or 3+5 in one launch when there is no LRU in between and the shapes allow
+    // attention launch of its own (token-major codes always; head-major codes behind an LRU table)
     attn_args aa{};
     aa.q = rope ? p.q_rot : p.q; aa.out = p.out; aa.dtype = p.dtype; aa.B = p.B; aa.QH = p.QH; aa.KH = p.KH; aa.k = p.k;
     aa.rows = 0; aa.scale = 0.f; aa.q_stride_b = static_cast<int64_t>(p.QH) * p.d;
@@ -269,17 +219,73 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     aa.keys = p.keys; aa.vals = p.vals; aa.idx = p.idx;
     aa.kv_stride_b = p.n_cap * p.KH * p.d; aa.kv_stride_h = p.d;
     aa.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
-    const bool both = (stages & SL_STAGE_SELECT) && (stages & SL_STAGE_ATTN);
-    // The fused tail attends per 4096-token block.  With few blocks and many kept
-    // rows each workgroup would gather hundreds of rows by itself; the separate
-    // attention launch cuts the rows into more runs than there are blocks then.
-    const int64_t tail_blocks = (p.n_max + 4095) / 4096;
-    const bool fuse_tail = g_fuse_select_attend == 2 || (g_fuse_select_attend == 1 && p.k <= 128 * tail_blocks);
-    if (both && p.lru_C == 0 && fuse_tail && sl_select_attend_supported(ta, aa))
-        return sl_select_attend_launch(ta, aa, ws + L.attn, attn_bytes, s);
-    if (stages & SL_STAGE_SELECT) {
-        rc = sl_select_launch(ta, s);
-        if (rc != SL_OK) return rc;
+    if (p.codes_head_major) {
+        // hash, then scorer + selection (+ attention, unless an LRU table update comes in between) as ONE
+        // launch over head-major codes
+        SL_REQUIRE(sl_fused_step_supported(G, W, G * p.nbits + 1, p.n_max, p.B, p.KH), SL_ERR_UNSUPPORTED);
+        const bool attend = p.lru_C == 0;
+        const int one = SL_STAGE_SCORE | SL_STAGE_SELECT | (attend ? SL_STAGE_ATTN : 0);
+        SL_REQUIRE((stages & one) == 0 || (stages & one) == one, SL_ERR_UNSUPPORTED);
+        ha.len_out = n_rows;
+        if (stages & SL_STAGE_HASH) {
+            rc = sl_hash_launch(ha, s);
+            if (rc != SL_OK) return rc;
+        }
+        if (stages & one) {
+            fused_args fa{};
+            fa.q_code = q_code; fa.k_code = p.codes; fa.q_stride_b = static_cast<int64_t>(p.QH) * W;
+            fa.k_stride_b = p.n_cap * p.KH * W; fa.k_stride_h = p.n_cap * W; fa.head_map = p.head_map;
+            select_args fs{};
+            fs.B = p.B; fs.KH = p.KH; fs.n_bins = G * p.nbits + 1; fs.idx = p.idx; fs.seq_lens = n_rows;
+            fs.k = p.k; fs.len_bias = 0; fs.n = p.n_max;
+            rc = sl_fused_step_launch(fa, fs, aa, attend, ws + L.fused, ws + L.attn, attn_bytes, s);
+            if (rc != SL_OK || attend) return rc;
+        }
+        if (attend) return SL_OK;
+    }
+    if (!p.codes_head_major) {
+        select_args ta{};
+        ta.B = p.B; ta.KH = p.KH; ta.n_bins = G * p.nbits + 1;
+        sl_select_carve(ta, ws + L.select, p.n_cap);
+        ta.hist_used = sl_select_hist_used(ta, p.n_max);
+        // the scorer of this step starts from a clean histogram: per (b, kv head) the copies this launch can reach
+        ha.zero_words = ta.hist;
+        ha.zero_rows = p.B * p.KH;
+        ha.zero_count = static_cast<int64_t>(ta.n_bins) * ta.hist_used;
+        ha.zero_stride = static_cast<int64_t>(ta.n_bins) * ta.hist_groups;
+        ha.len_out = n_rows;
+        // 2. score seq_lens[b] + 1 rows
+        hamming_args sa{};
+        sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.hist_span = ta.hist_span; sa.seq_lens = n_rows;
+        sa.B = p.B; sa.KH = p.KH; sa.G = G; sa.W = W; sa.head_map = p.head_map;
+        sa.n_bins = G * p.nbits + 1; sa.len_bias = 0; sa.n = p.n_max; sa.n_cap = p.n_cap;
+        sa.q_stride_b = static_cast<int64_t>(p.QH) * W; sa.k_stride_b = p.n_cap * p.KH * W; sa.out_stride_b = 0;
+        if (stages & SL_STAGE_HASH) {
+            rc = sl_hash_launch(ha, s);
+            if (rc != SL_OK) return rc;
+        }
+        if (stages & SL_STAGE_SCORE) {
+            rc = sl_hamming_launch(sa, true, s);
+            if (rc != SL_OK) return rc;
+        }
+
+        // 3. select
+        ta.score = score; ta.idx = p.idx; ta.seq_lens = n_rows;
+        ta.k = p.k; ta.len_bias = 0; ta.n = p.n_max;
+        ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
+        // 3. select -- or 3+5 in one launch when there is no LRU in between and the shapes allow
+        const bool both = (stages & SL_STAGE_SELECT) && (stages & SL_STAGE_ATTN);
+        // The fused tail attends per 4096-token block.  With few blocks and many kept
+        // rows each workgroup would gather hundreds of rows by itself; the separate
+        // attention launch cuts the rows into more runs than there are blocks then.
+        const int64_t tail_blocks = (p.n_max + 4095) / 4096;
+        const bool fuse_tail = g_fuse_select_attend == 2 || (g_fuse_select_attend == 1 && p.k <= 128 * tail_blocks);
+        if (both && p.lru_C == 0 && fuse_tail && sl_select_attend_supported(ta, aa))
+            return sl_select_attend_launch(ta, aa, ws + L.attn, attn_bytes, s);
+        if (stages & SL_STAGE_SELECT) {
+            rc = sl_select_launch(ta, s);
+            if (rc != SL_OK) return rc;
+        }
     }
 
     // 4. optional LRU, 5. attention

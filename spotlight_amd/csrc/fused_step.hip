@@ -19,6 +19,8 @@
 // workgroup that gives up sets an error word and goes on, so the launch always drains.
 #include "fused_step.h"
 
+#include <string.h>
+
 #include "attn_core.h"
 #include "topk_core.h"
 
@@ -26,24 +28,26 @@ namespace {
 
 constexpr int FS_NW = 8;
 constexpr int FS_THREADS = FS_NW * 64;
-constexpr int FS_SLOTS = 8;                          // rows per lane: row = block*4096 + wave*512 + slot*64 + lane
-constexpr int FS_BLOCK = FS_THREADS * FS_SLOTS;      // 4096 rows
 constexpr int FS_MAX_BPT = 2;                        // histogram bins per lane (<= 1024 bins)
 constexpr uint32_t FS_SPIN_LIMIT = 1u << 22;
 
 static_assert(FS_MAX_PEERS == AT_MAX_SPLITS, "one attention run per block of rows");
-static_assert(FS_BLOCK == 4096, "block of rows");
 
-template <typename T, int G>
+// FS_SLOTS rows per lane (row = block start + wave * 64 FS_SLOTS + slot * 64 + lane): blocks of 4096
+// rows, or of 8192 where 4096-row blocks would be more workgroups than the device holds at once.
+// ATTEND false: the launch ends with the list of kept rows (an LRU table update and the attention
+// launch follow); the block that reads its peers' histograms last lowers their flags.
+template <typename T, int G, int FS_SLOTS, bool ATTEND>
 __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_args fa, select_args sa, attn_args aa) {
     constexpr int W = 4;
+    constexpr int FS_BLOCK = FS_THREADS * FS_SLOTS;
     __shared__ uint32_t s_wave[64];
     __shared__ int s_tn[4];
     __shared__ uint32_t s_hist[FS_THREADS * FS_MAX_BPT];
     __shared__ uint32_t s_cnt[FS_NW];
     __shared__ int s_range[2];
     __shared__ int32_t s_list[FS_BLOCK];
-    __shared__ attn_shared<G, FS_NW> sh;
+    __shared__ attn_shared<ATTEND ? G : 1, FS_NW> sh;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -213,17 +217,33 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     // the list goes out with coalesced stores; the attention then runs over it
     __syncthreads();
     for (int i = tid; i < n_kept; i += FS_THREADS) out[first + i] = s_list[i];
-    attend_rows_and_merge<T, G, FS_NW>(aa, b, h, blk, S, s_list, n_kept, sh);
+    if constexpr (ATTEND) {
+        attend_rows_and_merge<T, G, FS_NW>(aa, b, h, blk, S, s_list, n_kept, sh);
+    } else {
+        // every lane of this block has used what it read from its peers (the barrier above): the last
+        // block of the head to get here lowers the flags for the next launch
+        if (S > 1 && wave == 0) {
+            uint32_t last = 0;
+            if (lane == 0) last = arrive_last(&aa.counter[bh], static_cast<uint32_t>(S)) ? 1u : 0u;
+            if (__builtin_amdgcn_readfirstlane(last)) {
+                if (lane < S) st_agent(fa.peer_flag + static_cast<int64_t>(bh) * FS_MAX_PEERS + lane, 0u);
+                if (lane == 0) st_agent(&aa.counter[bh], 0u);
+            }
+        }
+    }
 }
 
+int g_fused_rows = 0;  // sl_tune("fused_rows", 0 | 4096 | 8192): rows per block, 0 = 4096 while that fits the device
+
 // workgroups of the kernel the device holds at once (looked up once per flavour), <= 0 when unknown
-template <typename T, int G>
-int slots_tg() {
+template <typename T, int G, int SLOTS, bool ATTEND>
+int slots_of() {
     static int slots = 0;
     if (slots == 0) {
         int per_cu = 0, dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G>), FS_THREADS, 0) != hipSuccess) {
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                &per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G, SLOTS, ATTEND>), FS_THREADS, 0) != hipSuccess) {
             (void)hipGetLastError();
             return 0;
         }
@@ -232,33 +252,44 @@ int slots_tg() {
     return slots;
 }
 
-template <typename T>
-int slots_t(int G) {
-    switch (G) {
-        case 1: return slots_tg<T, 1>();
-        case 2: return slots_tg<T, 2>();
-        case 4: return slots_tg<T, 4>();
-        default: return -1;
+// Blocks of 4096 rows while all of them fit the device, else of 8192; every workgroup must be able
+// to be resident at once, because workgroups wait for their peers.
+template <typename T, int G, bool ATTEND>
+int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, hipStream_t s) {
+    const int64_t heads = static_cast<int64_t>(aa.B) * aa.KH;
+    const int64_t n = sa.n > 0 ? sa.n : 1;
+    const int64_t b8 = (n + 4095) / 4096, b16 = (n + 8191) / 8192;
+    const int s8 = slots_of<T, G, 8, ATTEND>();
+    if (s8 == 0) return SL_ERR_LAUNCH;
+    if (g_fused_rows != 8192 && b8 <= FS_MAX_PEERS && heads * b8 <= s8) {
+        score_select_attend_kernel<T, G, 8, ATTEND><<<dim3(static_cast<unsigned>(b8), aa.KH, aa.B), dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
+        return sl_check_launch();
     }
-}
-
-template <typename T, int G>
-int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
-    // every workgroup must be able to be resident at once: workgroups wait for their peers
-    const int slots = slots_tg<T, G>();
-    if (slots == 0) return SL_ERR_LAUNCH;
-    SL_REQUIRE(slots > 0 && static_cast<int64_t>(grid.x) * grid.y * grid.z <= slots, SL_ERR_UNSUPPORTED);
-    score_select_attend_kernel<T, G><<<grid, dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
+    const int s16 = slots_of<T, G, 16, ATTEND>();
+    if (s16 == 0) return SL_ERR_LAUNCH;
+    SL_REQUIRE(g_fused_rows != 4096 && b16 <= FS_MAX_PEERS && heads * b16 <= s16, SL_ERR_UNSUPPORTED);
+    score_select_attend_kernel<T, G, 16, ATTEND><<<dim3(static_cast<unsigned>(b16), aa.KH, aa.B), dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
     return sl_check_launch();
 }
 
 template <typename T>
-int launch_t(const fused_args &fa, const select_args &sa, const attn_args &aa, dim3 grid, hipStream_t s) {
+int launch_t(const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s) {
     switch (aa.QH / aa.KH) {
-        case 1: return launch_tg<T, 1>(fa, sa, aa, grid, s);
-        case 2: return launch_tg<T, 2>(fa, sa, aa, grid, s);
-        case 4: return launch_tg<T, 4>(fa, sa, aa, grid, s);
+        case 1: return attend ? launch_tg<T, 1, true>(fa, sa, aa, s) : launch_tg<T, 1, false>(fa, sa, aa, s);
+        case 2: return attend ? launch_tg<T, 2, true>(fa, sa, aa, s) : launch_tg<T, 2, false>(fa, sa, aa, s);
+        case 4: return attend ? launch_tg<T, 4, true>(fa, sa, aa, s) : launch_tg<T, 4, false>(fa, sa, aa, s);
         default: return SL_ERR_UNSUPPORTED;
+    }
+}
+
+template <typename T>
+int slots_t(int G, int rows, bool attend) {
+    const bool big = rows == 8192;
+    switch (G) {
+        case 1: return attend ? (big ? slots_of<T, 1, 16, true>() : slots_of<T, 1, 8, true>()) : (big ? slots_of<T, 1, 16, false>() : slots_of<T, 1, 8, false>());
+        case 2: return attend ? (big ? slots_of<T, 2, 16, true>() : slots_of<T, 2, 8, true>()) : (big ? slots_of<T, 2, 16, false>() : slots_of<T, 2, 8, false>());
+        case 4: return attend ? (big ? slots_of<T, 4, 16, true>() : slots_of<T, 4, 8, true>()) : (big ? slots_of<T, 4, 16, false>() : slots_of<T, 4, 8, false>());
+        default: return -1;
     }
 }
 
@@ -270,23 +301,28 @@ size_t sl_fused_ws_bytes(int B, int KH) {
            sl_align_up(sizeof(uint32_t) * bh * FS_MAX_PEERS * FS_NB_PAD, 256);       // published histograms
 }
 
-int sl_fused_step_slots(int dtype, int G) {
+int sl_fused_tune(const char *key, int value) {
+    if (!strcmp(key, "fused_rows") && (value == 0 || value == 4096 || value == 8192)) { g_fused_rows = value; return SL_OK; }
+    return SL_ERR_UNSUPPORTED;
+}
+
+int sl_fused_step_slots(int dtype, int G, int rows, bool attend) {
+    if (rows != 4096 && rows != 8192) return -1;
     switch (dtype) {
-        case SL_F32: return slots_t<float>(G);
-        case SL_BF16: return slots_t<bf16_t>(G);
-        case SL_F16: return slots_t<f16_t>(G);
+        case SL_F32: return slots_t<float>(G, rows, attend);
+        case SL_BF16: return slots_t<bf16_t>(G, rows, attend);
+        case SL_F16: return slots_t<f16_t>(G, rows, attend);
         default: return -1;
     }
 }
 
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH) {
-    const int64_t blocks = (n + FS_BLOCK - 1) / FS_BLOCK;
     return (G == 1 || G == 2 || G == 4) && W == 4 && n_bins <= FS_THREADS * FS_MAX_BPT && n_bins <= FS_NB_PAD &&
-           blocks <= FS_MAX_PEERS && B <= 65535 && KH <= 65535;
+           (n + 8191) / 8192 <= FS_MAX_PEERS && B <= 65535 && KH <= 65535;
 }
 
-int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, void *fused_ws, void *attn_ws, size_t attn_ws_bytes,
-                         hipStream_t s) {
+int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool attend, void *fused_ws, void *attn_ws,
+                         size_t attn_ws_bytes, hipStream_t s) {
     const int G = aa.QH / aa.KH;
     SL_REQUIRE(sl_fused_step_supported(G, 4, sa.n_bins, sa.n, aa.B, aa.KH), SL_ERR_UNSUPPORTED);
     SL_REQUIRE(fa.q_code && fa.k_code && fused_ws && sa.seq_lens, SL_ERR_NULL);
@@ -299,13 +335,10 @@ int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, void *fuse
     fa.error = fa.peer_flag + bh * FS_MAX_PEERS;
     fa.peer_hist = reinterpret_cast<uint32_t *>(static_cast<char *>(fused_ws) + sl_align_up(sizeof(uint32_t) * (bh * FS_MAX_PEERS + 64), 256));
     aa.peer_flag = fa.peer_flag;
-    int64_t blocks = (sa.n + FS_BLOCK - 1) / FS_BLOCK;
-    if (blocks < 1) blocks = 1;
-    const dim3 grid(static_cast<unsigned>(blocks), aa.KH, aa.B);
     switch (aa.dtype) {
-        case SL_F32: return launch_t<float>(fa, sa, aa, grid, s);
-        case SL_BF16: return launch_t<bf16_t>(fa, sa, aa, grid, s);
-        case SL_F16: return launch_t<f16_t>(fa, sa, aa, grid, s);
+        case SL_F32: return launch_t<float>(fa, sa, aa, attend, s);
+        case SL_BF16: return launch_t<bf16_t>(fa, sa, aa, attend, s);
+        case SL_F16: return launch_t<f16_t>(fa, sa, aa, attend, s);
         default: return SL_ERR_UNSUPPORTED;
     }
 }

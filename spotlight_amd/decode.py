@@ -93,17 +93,21 @@ class LayerDecodeState:
         B, QH, KH, d, W = self.B, self.QH, self.KH, self.d, self.W
         # Key codes: token-major [B, n_cap, KH, W] (the reference's layout, attn_k4_q28.cu:55) for the
         # three-launch step, or head-major [B, KH, n_cap, W] for the step whose scorer, selection and
-        # attention are ONE launch (a workgroup then owns 4096 contiguous rows of one kv head).  "auto"
+        # attention are ONE launch (a workgroup then owns 4096 or 8192 contiguous rows of one kv head;
+        # with an LRU table the launch ends at the selection).  "auto"
         # takes head-major whenever that launch covers the shape.  ``codes`` is always indexed
         # [b, row, kv head, word]; with head-major storage it is a strided view.
         if codes_layout == "auto":
-            blocks = (n_cap + 4095) // 4096
+            # without an LRU table the launch also attends, one run per block: keep <= 128 rows per 4096
+            # (and stay with the three launches beyond 64k rows: measured no faster there)
+            rows_ok = bool(lru_slots) or (k <= 128 * ((n_cap + 4095) // 4096) and n_cap <= 65536)
             fits = 0
-            if not lru_slots and QH // KH in (1, 2, 4) and W == 4 and n_cap <= 65536 and k <= 128 * blocks:
-                # all blocks of a launch must be resident at once; the library knows how many the device holds
+            if rows_ok and W == 4:
+                # all blocks of a launch must be resident at once; the library knows what the device holds
                 with torch.cuda.device(dev):
-                    fits = _lib.load().sl_decode_head_major_blocks(K._DTYPES[self.dtype], QH, KH)
-            codes_layout = "head" if B * KH * blocks <= fits else "token"
+                    fits = _lib.load().sl_decode_head_major_fits(K._DTYPES[self.dtype], B, QH, KH, self.nbits, n_cap,
+                                                                 int(bool(lru_slots)))
+            codes_layout = "head" if fits > 0 else "token"
         assert codes_layout in ("token", "head")
         self.codes_layout = codes_layout
         if codes_layout == "head":

@@ -134,13 +134,13 @@ def test_decode_ragged_batch(env):
         assert np.abs(out[b:b + 1] - want).max() <= 1e-5
 
 
-@pytest.mark.parametrize("lru", [0, 64])
-def test_decode_graph_replay_equals_eager(env, lru):
+@pytest.mark.parametrize("lru,layout", [(0, "auto"), (0, "token"), (64, "token"), (64, "head")])
+def test_decode_graph_replay_equals_eager(env, lru, layout):
     """A captured step replayed while the cache grows gives what eager steps give
     (also with the LRU table, whose misses the attention launch fetches)."""
     decode, kernel = env
     dtype = torch.bfloat16
-    states = [_make_state(decode, _gen(90), 2, 32, 8, 500, 640, 30, dtype, lru=lru) for _ in range(2)]
+    states = [_make_state(decode, _gen(90), 2, 32, 8, 500, 640, 30, dtype, lru=lru, codes_layout=layout) for _ in range(2)]
     eager, graphed = states
     graphed.capture(steps_ahead=8)
     g = _gen(91)
@@ -250,8 +250,8 @@ def test_lru_matches_bruteforce_model(env, C, k, n0, steps):
         n += 1
 
 
-@pytest.mark.parametrize("fuse", [0, 1])
-def test_decode_with_lru_gives_identical_attention(env, fuse):
+@pytest.mark.parametrize("fuse,layout", [(0, "token"), (1, "token"), (0, "head"), (1, "head")])
+def test_decode_with_lru_gives_identical_attention(env, fuse, layout):
     """The LRU layer changes where rows are read from, never the result.  With the
     two-launch tail (fuse=0) both states run the same attention kernel on the same rows
     in the same order and must agree bit for bit; with the fused tail the plain state
@@ -263,7 +263,7 @@ def test_decode_with_lru_gives_identical_attention(env, fuse):
     _lib.check(L.sl_tune(b"fuse_select_attend", fuse), "sl_tune")
     try:
         plain = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype, codes_layout="token")
-        lru = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype, lru=64)
+        lru = _make_state(decode, _gen(60), 2, 32, 8, 900, 1024, 40, dtype, lru=64, codes_layout=layout)
         models = [[orc.LruModel(64) for _ in range(8)] for _ in range(2)]
         g = _gen(61)
         for step in range(1, 9):
@@ -333,6 +333,44 @@ def test_decode_many_blocks_and_long_cache(env):
             _check_step(kernel, st, q, kn, vn, out, n0 + step, torch.bfloat16)
 
 
+@pytest.mark.parametrize("rows", [4096, 8192])
+@pytest.mark.parametrize("lru", [0, 512])
+def test_head_major_blocks_of_4096_and_8192_rows(env, rows, lru):
+    """Head-major codes with several blocks per (b, kv head), in both block sizes, without and with
+    the LRU table (where the launch ends at the selection and lowers its own flags): every step
+    equals the oracle and the state with token-major codes, over a block boundary."""
+    decode, kernel = env
+    from spotlight_amd import _lib
+    L = _lib.load()
+    dtype = torch.bfloat16
+    B, QH, KH, k = 2, 8, 2, 150
+    n0 = 2 * rows - 3          # the third step starts a new block
+    n_cap = (n0 + 64 + 7) // 8 * 8
+    _lib.check(L.sl_tune(b"fused_rows", rows), "sl_tune")
+    try:
+        head = _make_state(decode, _gen(80), B, QH, KH, n0, n_cap, k, dtype, lru=lru, codes_layout="head")
+        token = _make_state(decode, _gen(80), B, QH, KH, n0, n_cap, k, dtype, lru=lru, codes_layout="token")
+        g = _gen(81)
+        for step in range(6):
+            q = torch.randn(B, QH, 128, generator=g).to(dtype)
+            kn = torch.randn(B, KH, 128, generator=g).to(dtype)
+            vn = torch.randn(B, KH, 128, generator=g).to(dtype)
+            out = head.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).clone()
+            ref = token.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).clone()
+            assert not head.peer_wait_failed()
+            assert torch.equal(head.idx, token.idx), step
+            assert torch.equal(head.seq_lens, token.seq_lens)
+            if lru:   # same attention launch on the same rows
+                assert torch.equal(out, ref), step
+                assert torch.equal(head.slot_token, token.slot_token) and torch.equal(head.slot_stamp, token.slot_stamp)
+            else:
+                assert (out.float() - ref.float()).abs().max() <= 2e-2, step
+            if step in (0, 3):
+                _check_step(kernel, head, q, kn, vn, out, n0 + step, dtype)
+    finally:
+        _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
+
+
 def _random_cases(count, seed):
     import random
     rnd = random.Random(seed)
@@ -369,7 +407,8 @@ def test_decode_step_random_shapes(env, B, QH, KH, n0, k, dtype, kind, layout):
         _check_step(kernel, st, q, k_new, v_new, out, n0 + step, dtype)
 
 
-def test_budget_changes_on_a_live_lru_state(env):
+@pytest.mark.parametrize("layout", ["token", "head"])
+def test_budget_changes_on_a_live_lru_state(env, layout):
     """k lowered and raised between steps on one workspace, with the LRU table on and more than
     one attention run per (b, kv head): the arrival tickets must stay where they are (and zero)
     whatever k is, so every step still matches the oracle and the state without a table."""
@@ -377,7 +416,7 @@ def test_budget_changes_on_a_live_lru_state(env):
     dtype = torch.bfloat16
     B, QH, KH, n0, k_max = 2, 32, 8, 900, 100
     plain = _make_state(decode, _gen(70), B, QH, KH, n0, 1024, k_max, dtype)
-    lru = _make_state(decode, _gen(70), B, QH, KH, n0, 1024, k_max, dtype, lru=128)
+    lru = _make_state(decode, _gen(70), B, QH, KH, n0, 1024, k_max, dtype, lru=128, codes_layout=layout)
     g = _gen(71)
     n = n0
     for step, k in enumerate([100, 37, 100, 64, 12, 100, 99]):
