@@ -59,6 +59,8 @@ int sl_version(void);
  * workgroup instead of 4 (default 128);
  * "attn_mfma": 1 puts the q.K products of the attention on the matrix cores
  * (16-bit inputs; default 0: packed dot products and a lane butterfly);
+ * "fused_rows": rows per block of the step over head-major codes (4096, 8192;
+ * 0 = 4096 while all blocks are resident at once, the default);
  * "hist_copies": copies of the score histogram (4, 8, 16 or 32; 0 = by cache
  * length), to be set before any workspace is sized. */
 int sl_tune(const char *key, int value);
@@ -277,9 +279,10 @@ typedef struct {
     const void *w1_q, *b1_q, *w2_q, *b2_q;   /* [QH, ...]                       */
     const void *w1_k, *b1_k, *w2_k, *b2_k;   /* [KH, ...]                       */
     /* caches, token-major; codes_head_major != 0: codes are [B, KH, n_cap, W]  */
-    /* and scorer, selection and attention run as ONE launch (needs no LRU,     */
-    /* W == 4, QH/KH in {1,2,4}, n_max <= 65536 and a grid that fits the device */
-    /* at once: otherwise SL_ERR_UNSUPPORTED, use token-major codes)            */
+    /* and scorer, selection and (without an LRU table) attention run as ONE    */
+    /* launch; needs W == 4, QH/KH in {1,2,4}, n_max <= 131072 and a grid that  */
+    /* fits the device at once (sl_decode_head_major_fits): otherwise           */
+    /* SL_ERR_UNSUPPORTED, use token-major codes                                */
     int codes_head_major;
     uint32_t *codes;        /* [B, n_cap, KH, W]                                */
     void *keys, *vals;      /* [B, n_cap, KH, d]                                */
