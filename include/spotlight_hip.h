@@ -61,6 +61,10 @@ int sl_version(void);
  * (16-bit inputs; default 0: packed dot products and a lane butterfly);
  * "fused_rows": rows per block of the step over head-major codes (4096, 8192;
  * 0 = 4096 while all blocks are resident at once, the default);
+ * "fused_spin_limit", "fused_phantom_peer": for testing the bounded wait of that
+ * step -- polls before a workgroup gives up (0 = the default, 2^22) and 1 = every
+ * head also waits for a block that does not exist, so that each workgroup gives
+ * up after the limit, sets the error word and the launch still drains;
  * "hist_copies": copies of the score histogram (4, 8, 16 or 32; 0 = by cache
  * length), to be set before any workspace is sized. */
 int sl_tune(const char *key, int value);

@@ -21,6 +21,8 @@
 
 #include <string.h>
 
+#include <atomic>
+
 #include "attn_core.h"
 #include "topk_core.h"
 
@@ -29,7 +31,7 @@ namespace {
 constexpr int FS_NW = 8;
 constexpr int FS_THREADS = FS_NW * 64;
 constexpr int FS_MAX_BPT = 2;                        // histogram bins per lane (<= 1024 bins)
-constexpr uint32_t FS_SPIN_LIMIT = 1u << 22;
+constexpr uint32_t FS_SPIN_LIMIT = 1u << 22;   // polls a workgroup waits for a peer before it gives up (fused_args::spin_limit)
 
 static_assert(FS_MAX_PEERS == AT_MAX_SPLITS, "one attention run per block of rows");
 
@@ -124,10 +126,10 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
         if (tid == 0) st_agent(flags + blk, 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo));
         if (wave == 0) {
             uint32_t f = 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo);
-            if (lane < S) {
+            if (lane < S + fa.phantom_peers) {   // (phantom_peers: a flag nobody raises, to exercise the bounded wait)
                 uint32_t spins = 0;
                 while (((f = ld_agent(flags + lane)) & 0x80000000u) == 0u) {
-                    if (++spins > FS_SPIN_LIMIT) { st_agent(fa.error, 1u); f = 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo); break; }
+                    if (++spins > fa.spin_limit) { st_agent(fa.error, 1u); f = 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo); break; }
                     __builtin_amdgcn_s_sleep(1);
                 }
             }
@@ -234,21 +236,32 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
 }
 
 int g_fused_rows = 0;  // sl_tune("fused_rows", 0 | 4096 | 8192): rows per block, 0 = 4096 while that fits the device
+// sl_tune("fused_spin_limit", polls) and sl_tune("fused_phantom_peer", 0 | 1): for the test of the bounded
+// wait -- a short limit and a peer that does not exist make every workgroup give up and report it
+uint32_t g_fused_spin_limit = FS_SPIN_LIMIT;
+int g_fused_phantom_peer = 0;
 
-// workgroups of the kernel the device holds at once (looked up once per flavour), <= 0 when unknown
+// workgroups of the kernel the CURRENT device holds at once (looked up once per flavour and device;
+// any thread may ask), 0 when the runtime cannot tell, -1 when the kernel does not fit at all
 template <typename T, int G, int SLOTS, bool ATTEND>
 int slots_of() {
-    static int slots = 0;
-    if (slots == 0) {
-        int per_cu = 0, dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                &per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G, SLOTS, ATTEND>), FS_THREADS, 0) != hipSuccess) {
-            (void)hipGetLastError();
-            return 0;
-        }
-        slots = per_cu * cus > 0 ? per_cu * cus : -1;
+    constexpr int MAX_DEV = 64;
+    static std::atomic<int> cache[MAX_DEV];   // 0 = not looked up yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    if (dev >= 0 && dev < MAX_DEV) {
+        const int known = cache[dev].load(std::memory_order_relaxed);
+        if (known != 0) return known;
     }
+    int per_cu = 0, cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G, SLOTS, ATTEND>), FS_THREADS, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    const int slots = per_cu * cus > 0 ? per_cu * cus : -1;
+    if (dev >= 0 && dev < MAX_DEV) cache[dev].store(slots, std::memory_order_relaxed);
     return slots;
 }
 
@@ -303,6 +316,8 @@ size_t sl_fused_ws_bytes(int B, int KH) {
 
 int sl_fused_tune(const char *key, int value) {
     if (!strcmp(key, "fused_rows") && (value == 0 || value == 4096 || value == 8192)) { g_fused_rows = value; return SL_OK; }
+    if (!strcmp(key, "fused_spin_limit") && value >= 0) { g_fused_spin_limit = value ? static_cast<uint32_t>(value) : FS_SPIN_LIMIT; return SL_OK; }
+    if (!strcmp(key, "fused_phantom_peer") && (value == 0 || value == 1)) { g_fused_phantom_peer = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
 
@@ -335,6 +350,9 @@ int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool atten
     fa.error = fa.peer_flag + bh * FS_MAX_PEERS;
     fa.peer_hist = reinterpret_cast<uint32_t *>(static_cast<char *>(fused_ws) + sl_align_up(sizeof(uint32_t) * (bh * FS_MAX_PEERS + 64), 256));
     aa.peer_flag = fa.peer_flag;
+    fa.spin_limit = g_fused_spin_limit;
+    // (a phantom needs a free flag slot: heads that already have 16 blocks get none)
+    fa.phantom_peers = g_fused_phantom_peer && (sa.n + 4095) / 4096 < FS_MAX_PEERS ? 1 : 0;
     switch (aa.dtype) {
         case SL_F32: return launch_t<float>(fa, sa, aa, attend, s);
         case SL_BF16: return launch_t<bf16_t>(fa, sa, aa, attend, s);

@@ -371,6 +371,41 @@ def test_head_major_blocks_of_4096_and_8192_rows(env, rows, lru):
         _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
 
 
+@pytest.mark.parametrize("lru", [0, 256])
+def test_bounded_wait_gives_up_reports_and_drains(env, lru):
+    """The blocks of a head wait for each other's flags at most a fixed number of polls.  Forced
+    from the host -- every head also waits for a block that does not exist, with a short limit --
+    each workgroup gives up, the launch still finishes, the error word says so, and after the
+    workspace is cleared the state steps normally again."""
+    decode, kernel = env
+    from spotlight_amd import _lib
+    L = _lib.load()
+    dtype = torch.bfloat16
+    B, QH, KH, n0, k = 1, 8, 2, 9000, 100
+    st = _make_state(decode, _gen(85), B, QH, KH, n0, (n0 + 64 + 7) // 8 * 8, k, dtype, lru=lru, codes_layout="head")
+    g = _gen(86)
+    fresh = lambda: tuple(torch.randn(B, h, 128, generator=g).to(dtype) for h in (QH, KH, KH))
+    q, kn, vn = fresh()
+    out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).clone()
+    _check_step(kernel, st, q, kn, vn, out, n0, dtype)
+    _lib.check(L.sl_tune(b"fused_spin_limit", 64), "sl_tune")
+    _lib.check(L.sl_tune(b"fused_phantom_peer", 1), "sl_tune")
+    try:
+        q, kn, vn = fresh()
+        st.step(q.to(DEV), kn.to(DEV), vn.to(DEV))
+        torch.cuda.synchronize()          # the launch drained
+        assert st.peer_wait_failed()
+        assert st.seq_lens.cpu().tolist() == [n0 + 2] * B
+    finally:
+        _lib.check(L.sl_tune(b"fused_spin_limit", 0), "sl_tune")
+        _lib.check(L.sl_tune(b"fused_phantom_peer", 0), "sl_tune")
+    st.reset_workspace()
+    assert not st.peer_wait_failed()
+    q, kn, vn = fresh()
+    out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).clone()
+    _check_step(kernel, st, q, kn, vn, out, n0 + 2, dtype)
+
+
 def _random_cases(count, seed):
     import random
     rnd = random.Random(seed)
