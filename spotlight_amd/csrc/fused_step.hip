@@ -1,7 +1,8 @@
 // Scorer + count-select + sparse attention in ONE launch: the decode step's second and last launch
-// when the key codes are stored head-major.
+// when the key codes are stored head-major (behind an LRU table the launch ends at the selection).
 //
-// With codes laid out [B, KH, n_cap, W] a workgroup can own a block of 4096 rows of ONE (b, kv head):
+// With codes laid out [B, KH, n_cap, W] a workgroup can own a block of 4096 rows of ONE (b, kv head)
+// (8192 rows, 16 per lane, when that is what it takes for all blocks to be resident):
 // it streams the block's codes (64 KB, contiguous), keeps the 8 scores per lane in registers and
 // builds the block's score histogram in LDS.  The only thing it lacks for the selection is what the
 // other blocks of the same (b, kv head) saw, so the blocks -- at most 16, all resident at the same
@@ -16,7 +17,8 @@
 // Waiting on other workgroups is only safe while every workgroup of the launch can be resident at
 // once; the host checks the grid against the device's capacity for this kernel and otherwise the
 // caller must use the three-launch path (token-major codes).  The wait is bounded all the same: a
-// workgroup that gives up sets an error word and goes on, so the launch always drains.
+// workgroup that gives up sets an error word and goes on, so the launch always drains (exercised
+// from the host with a short limit and a peer that does not exist, sl_tune "fused_phantom_peer").
 #include "fused_step.h"
 
 #include <string.h>
