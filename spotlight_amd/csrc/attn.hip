@@ -2,7 +2,7 @@
 //
 // The step is latency bound (a few MB per layer), so the launch is organised
 // around memory round trips rather than around occupancy: the k selected rows
-// of a (batch, kv head) are cut into at most AT_MAX_SPLITS runs of `rows`
+// of a (batch, kv head) are cut into at most AT_PART_SPLITS runs of `rows`
 // consecutive ranks, one workgroup of 4 waves per run; the run's row numbers
 // are fetched into LDS in one go and the shared body (attn_core.h) does the
 // rest.
@@ -22,7 +22,7 @@ constexpr int AT_MAX_ROWS = 1024;    // rows per run (LDS row-number buffer)
 // the only part that has to stay zero between calls.
 constexpr size_t AT_COUNTER_BYTES = 64 * 1024;
 
-template <typename T, int G, int NW, bool FETCH, bool MF>
+template <typename T, int G, int NW, bool FETCH, bool MF, int MAXS>
 __global__ __launch_bounds__(NW * 64) void sparse_attn_kernel(attn_args a) {
     constexpr int AT_THREADS = NW * 64;
     __shared__ int s_row[AT_MAX_ROWS];
@@ -38,25 +38,31 @@ __global__ __launch_bounds__(NW * 64) void sparse_attn_kernel(attn_args a) {
         for (int i = threadIdx.x; i < a.rows; i += AT_THREADS) s_src[i] = r_lo + i < r_hi ? fetch[r_lo + i] : -1;
     }
     __syncthreads();
-    attend_rows_and_merge<T, G, NW, FETCH, MF>(a, b, h, split, gridDim.x, s_row, a.rows, sh, s_src);
+    attend_rows_and_merge<T, G, NW, FETCH, MF, MAXS>(a, b, h, split, gridDim.x, s_row, a.rows, sh, s_src);
 }
 
 int g_attn_wide_rows = AT_WIDE_ROWS;  // sl_tune("attn_wide_rows", n)
 int g_attn_mfma = 0;                  // sl_tune("attn_mfma", 0 | 1): score phase on the matrix cores (16-bit inputs)
 
-template <typename T, int G, bool MF>
-int launch_mf(const attn_args &a, hipStream_t s) {
-    const int S = (a.k + a.rows - 1) / a.rows;
+template <typename T, int G, bool MF, int MAXS>
+int launch_s(const attn_args &a, int S, hipStream_t s) {
     const dim3 grid(S, a.KH, a.B);
     const bool wide = a.rows >= g_attn_wide_rows;
     if (a.fetch) {
-        if (wide) sparse_attn_kernel<T, G, 8, true, MF><<<grid, dim3(512), 0, s>>>(a);
-        else sparse_attn_kernel<T, G, 4, true, MF><<<grid, dim3(256), 0, s>>>(a);
+        if (wide) sparse_attn_kernel<T, G, 8, true, MF, MAXS><<<grid, dim3(512), 0, s>>>(a);
+        else sparse_attn_kernel<T, G, 4, true, MF, MAXS><<<grid, dim3(256), 0, s>>>(a);
     } else {
-        if (wide) sparse_attn_kernel<T, G, 8, false, MF><<<grid, dim3(512), 0, s>>>(a);
-        else sparse_attn_kernel<T, G, 4, false, MF><<<grid, dim3(256), 0, s>>>(a);
+        if (wide) sparse_attn_kernel<T, G, 8, false, MF, MAXS><<<grid, dim3(512), 0, s>>>(a);
+        else sparse_attn_kernel<T, G, 4, false, MF, MAXS><<<grid, dim3(256), 0, s>>>(a);
     }
     return sl_check_launch();
+}
+
+template <typename T, int G, bool MF>
+int launch_mf(const attn_args &a, hipStream_t s) {
+    const int S = (a.k + a.rows - 1) / a.rows;
+    // the merge keeps one register per (output, run): the 32-run flavour only where it is needed
+    return S <= AT_MAX_SPLITS ? launch_s<T, G, MF, AT_MAX_SPLITS>(a, S, s) : launch_s<T, G, MF, AT_PART_SPLITS>(a, S, s);
 }
 
 template <typename T, int G>
@@ -83,14 +89,14 @@ int dispatch_g(const attn_args &a, hipStream_t s) {
 }
 
 // Rows per run: about one workgroup per compute unit over the whole launch,
-// never more than AT_MAX_SPLITS runs per (b, kv head), whole 64-row iterations.
+// never more than AT_PART_SPLITS runs per (b, kv head), whole 64-row iterations.
 int g_attn_target_wgs = 256;  // sl_tune("attn_target_wgs", n)
 
 int pick_rows(int B, int KH, int k) {
     const int64_t bh = static_cast<int64_t>(B) * KH;
     int64_t want = (g_attn_target_wgs + bh - 1) / bh;
     if (want < 1) want = 1;
-    if (want > AT_MAX_SPLITS) want = AT_MAX_SPLITS;
+    if (want > AT_PART_SPLITS) want = AT_PART_SPLITS;
     int rows = static_cast<int>((k + want - 1) / want);
     rows = (rows + AT_ITER_ROWS - 1) / AT_ITER_ROWS * AT_ITER_ROWS;
     return rows;
@@ -111,7 +117,7 @@ size_t sl_attn_ws_bytes(int B, int QH, int KH, int k) {
     if (B <= 0 || QH <= 0 || KH <= 0 || k <= 0) return 0;
     const size_t bh = static_cast<size_t>(B) * KH;
     const size_t G = static_cast<size_t>(QH / KH);
-    return AT_COUNTER_BYTES + sl_align_up(bh * AT_MAX_SPLITS * G * AT_PART * sizeof(float), 256);
+    return AT_COUNTER_BYTES + sl_align_up(bh * AT_PART_SPLITS * G * AT_PART * sizeof(float), 256);
 }
 
 int sl_attn_prepare(attn_args &a, void *ws, size_t ws_bytes) {
@@ -130,7 +136,7 @@ int sl_attn_launch(attn_args a, void *ws, size_t ws_bytes, hipStream_t s) {
     if (a.rows <= 0) a.rows = pick_rows(a.B, a.KH, a.k);
     if (a.fetch) SL_REQUIRE(a.src_keys && a.src_vals, SL_ERR_NULL);
     SL_REQUIRE(a.rows % AT_ITER_ROWS == 0 && a.rows <= AT_MAX_ROWS, SL_ERR_UNSUPPORTED);
-    SL_REQUIRE((a.k + a.rows - 1) / a.rows <= AT_MAX_SPLITS, SL_ERR_UNSUPPORTED);  // k <= 16384
+    SL_REQUIRE((a.k + a.rows - 1) / a.rows <= AT_PART_SPLITS, SL_ERR_UNSUPPORTED);  // k <= 32768
     switch (a.dtype) {
         case SL_F32: return dispatch_g<float>(a, s);
         case SL_BF16: return dispatch_g<bf16_t>(a, s);

@@ -31,7 +31,8 @@
 
 constexpr int AT_D = 128;
 constexpr int AT_PART = AT_D + 2;    // acc[128], m, l
-constexpr int AT_MAX_SPLITS = 16;    // runs per (b, kv head): the merge loads them all at once
+constexpr int AT_MAX_SPLITS = 16;    // runs per (b, kv head) where a run is a block of rows (select_attend, fused_step)
+constexpr int AT_PART_SPLITS = 32;   // run slots per (b, kv head) in the workspace; the stand-alone attention launch uses up to 32
 
 constexpr int DPP_ROW_MIRROR = 0x140;       // lane i <- lane 15 - i  (i ^ 15)
 constexpr int DPP_ROW_HALF_MIRROR = 0x141;  // lane i <- lane 7 - i within 8 lanes  (i ^ 7)
@@ -55,7 +56,7 @@ struct attn_shared {
     alignas(16) float acc[NW][G][AT_D];
     alignas(16) float l[NW][GP];
     float M[GP], L[G];
-    float w[AT_MAX_SPLITS][G];
+    float w[AT_PART_SPLITS][G];
     int last;
 };
 
@@ -208,7 +209,8 @@ template <int U> __device__ __forceinline__ float head_max(float v) {
 // s_src[i] >= 0 names a row of the source store that row s_row[i] is to be filled
 // from: the kernel reads that row instead, and writes the K slices / V pairs it
 // loaded to row s_row[i] of keys / vals after it has used them.
-template <typename T, int G, int NW, bool FETCH = false, bool MF = false>
+// MAXS: the most runs a (b, kv head) can have in this launch (16 or 32): the merge loads them all at once.
+template <typename T, int G, int NW, bool FETCH = false, bool MF = false, int MAXS = AT_MAX_SPLITS>
 __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b, int h, int split, int S,
                                                       const int *s_row, int n_rows, attn_shared<G, NW, MF> &sh,
                                                       const int *s_src = nullptr) {
@@ -426,7 +428,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
 
     const int bh = b * a.KH + h;
     T *ob = static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.QH + static_cast<int64_t>(h) * G) * AT_D;
-    float *part_out = a.part + (static_cast<int64_t>(bh) * AT_MAX_SPLITS + split) * G * AT_PART;
+    float *part_out = a.part + (static_cast<int64_t>(bh) * AT_PART_SPLITS + split) * G * AT_PART;
     if (S == 1) __syncthreads();  // sh.L is read below
     for (int e = tid; e < G * AT_D; e += NT) {
         const int g = e / AT_D, c = e % AT_D;
@@ -460,31 +462,32 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
     // merge the S runs by log-sum-exp.  All loads are issued together: the runs'
     // accumulators by every lane, their (max, sum) by one wave per head, which turns
     // them into one weight per (run, head) for everybody.
-    const float *pb = a.part + static_cast<int64_t>(bh) * AT_MAX_SPLITS * G * AT_PART;
+    const float *pb = a.part + static_cast<int64_t>(bh) * AT_PART_SPLITS * G * AT_PART;
     constexpr int PER = (G * AT_D + NT - 1) / NT;  // outputs per lane
-    float pa[PER][AT_MAX_SPLITS];
+    float pa[PER][MAXS];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const int e = tid + i * NT;
         const int g = (e < G * AT_D ? e : 0) / AT_D, c = e % AT_D;
 #pragma unroll
-        for (int sp = 0; sp < AT_MAX_SPLITS; ++sp) {
+        for (int sp = 0; sp < MAXS; ++sp) {
             float v = 0.f;
             if (sp < S) v = ld_agent(pb + (static_cast<int64_t>(sp) * G + g) * AT_PART + c);  // uniform: absent runs cost nothing
             pa[i][sp] = e < G * AT_D ? v : 0.f;
         }
     }
-    static_assert(AT_MAX_SPLITS == 16, "the runs of a head fit one 16-lane row");
+    static_assert(MAXS == 16 || MAXS == 32, "the runs of a head fit one 16-lane row, or half a wave");
     for (int g = wave; g < G; g += NW) {
-        // lanes 0 .. 15 hold one run each: reductions stay inside the 16-lane row
+        // lanes 0 .. MAXS - 1 hold one run each: with 16 runs the reductions stay inside a 16-lane row
         const int sp = lane < S ? lane : 0;
         const float *ps = pb + (static_cast<int64_t>(sp) * G + g) * AT_PART;
         const float mraw = ld_agent(ps + AT_D), lraw = ld_agent(ps + AT_D + 1);
         const float mine = lane < S ? mraw : -INFINITY;
-        const float M = row16_max(mine);
+        const float M = MAXS == 16 ? row16_max(mine) : wave_max(mine);
         const float w = mine == -INFINITY ? 0.f : __expf(mine - M);
-        const float L = row16_sum(lane < S ? lraw * w : 0.f);
-        if (lane < AT_MAX_SPLITS) sh.w[lane][g] = w;
+        const float lw = lane < S ? lraw * w : 0.f;
+        const float L = MAXS == 16 ? row16_sum(lw) : wave_sum(lw);
+        if (lane < MAXS) sh.w[lane][g] = w;
         if (lane == 0) sh.L[g] = L;
     }
     __syncthreads();
@@ -495,7 +498,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             const int g = e / AT_D;
             float O = 0.f;
 #pragma unroll
-            for (int sp = 0; sp < AT_MAX_SPLITS; ++sp) O = fmaf(pa[i][sp], sh.w[sp][g], O);
+            for (int sp = 0; sp < MAXS; ++sp) O = fmaf(pa[i][sp], sh.w[sp][g], O);
             const float L = sh.L[g];
             ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         }
