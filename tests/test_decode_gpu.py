@@ -372,6 +372,45 @@ def test_head_major_blocks_of_4096_and_8192_rows(env, rows, lru):
 
 
 @pytest.mark.parametrize("lru", [0, 256])
+@pytest.mark.parametrize("rows", [4096, 8192])
+def test_head_major_ragged_batch_with_different_block_counts(env, rows, lru):
+    """One batch whose sequences have 1, 2 and 3 blocks of rows (and one that ends exactly on a block
+    boundary, so the step opens a new block): every (b, kv head) swaps histograms among ITS blocks
+    only, blocks beyond a sequence's length drop out, and each sequence matches the oracle."""
+    decode, kernel = env
+    from spotlight_amd import _lib
+    L = _lib.load()
+    dtype = torch.bfloat16
+    B, QH, KH, k = 4, 8, 2, 120
+    lens = [rows // 2, rows, 2 * rows + 5, 3 * rows - 1]
+    n_cap = (3 * rows + 64 + 7) // 8 * 8
+    _lib.check(L.sl_tune(b"fused_rows", rows), "sl_tune")
+    try:
+        g = _gen(88)
+        st = _make_state(decode, g, B, QH, KH, 3 * rows, n_cap, k, dtype, lru=lru, codes_layout="head")
+        st.seq_lens.copy_(torch.tensor(lens, dtype=torch.int32))
+        for step in range(2):
+            q = torch.randn(B, QH, 128, generator=g).to(dtype)
+            kn = torch.randn(B, KH, 128, generator=g).to(dtype)
+            vn = torch.randn(B, KH, 128, generator=g).to(dtype)
+            out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV)).float().cpu().numpy()
+            assert not st.peer_wait_failed()
+            hq = st.hash_q
+            q_code = kernel.hash_mlp_pack(q.to(DEV), hq.w1, hq.b1, hq.w2, hq.b2).cpu().numpy()[:, None]
+            assert st.seq_lens.cpu().tolist() == [l + step + 1 for l in lens]
+            for b, l in enumerate(lens):
+                n = l + step + 1
+                codes = st.codes[b:b + 1, :n].cpu().numpy()
+                want_idx = orc.topk_stable(orc.hamming_score_u32(q_code[b:b + 1], codes, "blocked"), k)
+                np.testing.assert_array_equal(st.idx[b:b + 1].cpu().numpy(), want_idx)
+                want = orc.sparse_attention(q[b:b + 1].float().numpy(), st.keys[b:b + 1, :n].float().cpu().numpy(),
+                                            st.vals[b:b + 1, :n].float().cpu().numpy(), want_idx)
+                assert np.abs(out[b:b + 1] - want).max() <= 2e-2, (step, b)
+    finally:
+        _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
+
+
+@pytest.mark.parametrize("lru", [0, 256])
 def test_bounded_wait_gives_up_reports_and_drains(env, lru):
     """The blocks of a head wait for each other's flags at most a fixed number of polls.  Forced
     from the host -- every head also waits for a block that does not exist, with a short limit --
