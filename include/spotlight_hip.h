@@ -286,7 +286,10 @@ typedef struct {
     /* and scorer, selection and (without an LRU table) attention run as ONE    */
     /* launch; needs W == 4, QH/KH in {1,2,4}, n_max <= 131072 and a grid that  */
     /* fits the device at once (sl_decode_head_major_fits): otherwise           */
-    /* SL_ERR_UNSUPPORTED, use token-major codes                                */
+    /* SL_ERR_UNSUPPORTED, use token-major codes.  The blocks of that launch    */
+    /* wait for each other (bounded; see sl_decode_error_offset), which assumes */
+    /* the launch gets the whole device: with other kernels running at the same */
+    /* time on other streams prefer token-major codes                           */
     int codes_head_major;
     uint32_t *codes;        /* [B, n_cap, KH, W]                                */
     void *keys, *vals;      /* [B, n_cap, KH, d]                                */
