@@ -201,6 +201,24 @@ __device__ __forceinline__ void st_agent(uint32_t *p, uint32_t v) {
 __device__ __forceinline__ uint32_t ld_agent(const uint32_t *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Workgroups of a 1-D grid go to the device's 8 XCDs (each with its own L2) in turn: workgroup i
+// runs on XCD (i + c) % 8.  Work items that exchange data -- the parts of one group -- are therefore
+// numbered so that a group's parts share i % 8: their device-coherent stores and loads then meet in
+// one L2 (measured: publish + wait + read among 8 peers 0.6 us faster than with neighbouring ids;
+// used where it also measured faster in the kernel itself: the one-launch scorer + tail).
+// Group j sits in class j % 8 at position j / 8; class c owns the workgroups c, c + 8, c + 16, ...
+// and a position takes `parts` consecutive ones of them.  Results do not depend on the mapping.
+constexpr int SL_XCDS = 8;
+__host__ __device__ __forceinline__ unsigned xcd_grid(unsigned groups, unsigned parts) {
+    return SL_XCDS * ((groups + SL_XCDS - 1) / SL_XCDS) * parts;
+}
+// false: this workgroup has no work (groups not a multiple of 8)
+__device__ __forceinline__ bool xcd_unmap(unsigned wg, unsigned groups, unsigned parts, int &group, int &part) {
+    const unsigned c = wg % SL_XCDS, i = wg / SL_XCDS;
+    group = static_cast<int>(c + SL_XCDS * (i / parts));
+    part = static_cast<int>(i % parts);
+    return static_cast<unsigned>(group) < groups;
+}
 // all earlier memory operations of this lane have completed
 __device__ __forceinline__ void publish_wait() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");

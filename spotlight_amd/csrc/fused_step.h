@@ -15,6 +15,7 @@ struct fused_args {
     uint32_t *peer_flag;      // workspace: [B*KH][FS_MAX_PEERS], zero between launches
     uint32_t *error;          // workspace: set to 1 by a workgroup that gave up waiting for a peer
     uint32_t spin_limit;      // polls before giving up (set by the launcher)
+    unsigned blocks;          // blocks of rows per (b, kv head) the grid was sized for (set by the launcher)
     int phantom_peers;        // 0; 1 = also wait for a block that does not exist (test of the bounded wait)
 };
 
