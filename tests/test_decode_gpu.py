@@ -410,6 +410,49 @@ def test_head_major_ragged_batch_with_different_block_counts(env, rows, lru):
         _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
 
 
+def test_head_major_equals_token_major_on_random_shapes(env):
+    """Both code layouts are the same function of the same inputs: 200 seeded shapes (batch, heads, group
+    size, rows around the block boundaries, k, LRU table or not, dtype, block size), three steps each;
+    indices and lengths must be identical, outputs equal to rounding, and no wait may have run out."""
+    import random
+    decode, kernel = env
+    from spotlight_amd import _lib
+    L = _lib.load()
+    rnd = random.Random(2024)
+    try:
+        for case in range(200):
+            KH = rnd.choice([1, 2, 4, 8]); G = rnd.choice([1, 2, 4]); QH = KH * G
+            B = rnd.choice([1, 1, 2, 3, 5])
+            n0 = rnd.choice([1, 5, 63, 100, 1000, 4095, 4096, 4097, 8191, 8192, 8193, 12000, 12287, 12288, 16384, 20000])
+            k = rnd.choice([1, 7, 64, 100, 300, 600])
+            lru = rnd.choice([0, 0, 1024])
+            dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+            rows = rnd.choice([0, 4096, 8192])
+            n_cap = (n0 + 16 + 7) // 8 * 8
+            cg = torch.Generator().manual_seed(case)
+            g = torch.Generator(device=DEV).manual_seed(case)
+            hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, DEV, cg)
+            hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, DEV, cg)
+            kk = torch.randn((B, n0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+            vv = torch.randn((B, n0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+            head, token = (decode.LayerDecodeState(B, QH, KH, 128, n_cap, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru,
+                                                   codes_layout=layout) for layout in ("head", "token"))
+            head.prefill(kk, vv)
+            token.prefill(kk, vv)
+            _lib.check(L.sl_tune(b"fused_rows", rows), "sl_tune")
+            what = (case, B, QH, KH, n0, k, lru, dtype, rows)
+            for step in range(3):
+                q, kn, vn = (torch.randn((B, h, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype) for h in (QH, KH, KH))
+                a = head.step(q, kn, vn).float().clone()
+                b = token.step(q, kn, vn).float().clone()
+                assert torch.equal(head.idx, token.idx), (what, step)
+                assert torch.equal(head.seq_lens, token.seq_lens), (what, step)
+                assert not head.peer_wait_failed(), (what, step)
+                assert (a - b).abs().max().item() <= TOL[dtype], (what, step)
+    finally:
+        _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
+
+
 @pytest.mark.parametrize("lru", [0, 256])
 def test_bounded_wait_gives_up_reports_and_drains(env, lru):
     """The blocks of a head wait for each other's flags at most a fixed number of polls.  Forced
