@@ -73,6 +73,9 @@ def main():
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS) + ["c5"])
     ap.add_argument("--layers", type=int, default=None)
     ap.add_argument("--batch", type=int, default=None, help="override the configuration's batch size (c1-c4)")
+    ap.add_argument("--context", type=int, default=None,
+                    help="override the configuration's context length (c1-c4); k follows as 2 %% of it unless --keep is given")
+    ap.add_argument("--keep", type=int, default=None, help="override k, the rows kept per (batch entry, kv head)")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch heuristic passed to sl_tune (e.g. attn_target_wgs=128)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -104,6 +107,13 @@ def main():
     if args.batch:
         c["B"] = args.batch
         c["desc"] += f", batch overridden to {args.batch}"
+    if args.context:
+        c["n0"] = args.context
+        c["k"] = max(1, args.context - int(args.context * 0.98))
+        c["desc"] += f", context overridden to {args.context} (k = {c['k']})"
+    if args.keep:
+        c["k"] = args.keep
+        c["desc"] += f", k overridden to {args.keep}"
     L = args.layers or c["layers"]
     steps = args.steps if args.steps is not None else (256 if args.config == "c3" else 1000)
     warmup = args.warmup if args.warmup is not None else 64

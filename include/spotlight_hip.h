@@ -321,11 +321,11 @@ size_t sl_decode_workspace_bytes(const sl_decode_params *p);
 size_t sl_decode_error_offset(const sl_decode_params *p);
 /* 1 if sl_decode_step can run this shape over head-major codes on the current
  * device, 0 if not (the caller then keeps token-major codes), negative on bad
- * arguments.  The blocks of rows of such a launch (4096 rows, or 8192 when that is
- * what fits) wait for each other, so B * KH * blocks may not exceed the workgroups
+ * arguments.  The blocks of rows of such a launch (4096 rows; 8192 when that is
+ * what fits; 2048 or 1024 when a short context keeps many rows) wait for each other, so B * KH * blocks may not exceed the workgroups
  * the device holds at once; n_max is the largest row bound the caller will pass
  * (its n_cap).  No counterpart in the reference. */
-int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int with_lru);
+int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int k, int with_lru);
 int sl_decode_step(const sl_decode_params *p, void *stream);
 
 /* The same step restricted to a subset of its kernels, for profiling one

@@ -65,7 +65,7 @@ SIGNATURES = {
     "sl_sparse_gqa_attn": (c_int, [c_void_p] * 5 + [c_int] * 6 + [c_int64] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),
     "sl_decode_workspace_bytes": (c_size_t, [C.POINTER(DecodeParams)]),
     "sl_decode_error_offset": (c_size_t, [C.POINTER(DecodeParams)]),
-    "sl_decode_head_major_fits": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int64, c_int]),
+    "sl_decode_head_major_fits": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int64, c_int, c_int]),
     "sl_decode_step": (c_int, [C.POINTER(DecodeParams), c_void_p]),
     "sl_decode_stages": (c_int, [C.POINTER(DecodeParams), c_int, c_void_p]),
     "sl_probe_launch": (c_int, [c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),

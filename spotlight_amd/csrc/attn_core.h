@@ -31,7 +31,7 @@
 
 constexpr int AT_D = 128;
 constexpr int AT_PART = AT_D + 2;    // acc[128], m, l
-constexpr int AT_MAX_SPLITS = 16;    // runs per (b, kv head) where a run is a block of rows (select_attend, fused_step)
+constexpr int AT_MAX_SPLITS = 16;    // runs per (b, kv head) of the 16-run merge flavour (select_attend; the default of the others)
 constexpr int AT_PART_SPLITS = 32;   // run slots per (b, kv head) in the workspace; the stand-alone attention launch uses up to 32
 
 constexpr int DPP_ROW_MIRROR = 0x140;       // lane i <- lane 15 - i  (i ^ 15)
@@ -503,7 +503,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         }
     }
-    if (a.peer_flag && tid < S) st_agent(&a.peer_flag[static_cast<int64_t>(bh) * AT_MAX_SPLITS + tid], 0u);
+    if (a.peer_flag && tid < S) st_agent(&a.peer_flag[static_cast<int64_t>(bh) * AT_PART_SPLITS + tid], 0u);
     if (tid == 0) {
         st_agent(&a.counter[bh], 0u);
         if (a.bump_lens && h == 0) a.bump_lens[b] += 1;

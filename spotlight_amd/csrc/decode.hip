@@ -147,14 +147,11 @@ extern "C" size_t sl_decode_error_offset(const sl_decode_params *p) {
     return layout(*p).fused + sizeof(uint32_t) * static_cast<size_t>(p->B) * p->KH * FS_MAX_PEERS;
 }
 
-extern "C" int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int with_lru) {
-    SL_REQUIRE(B > 0 && QH > 0 && KH > 0 && QH % KH == 0 && nbits > 0 && nbits % 32 == 0 && n_max > 0, SL_ERR_SHAPE);
+extern "C" int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int k, int with_lru) {
+    SL_REQUIRE(B > 0 && QH > 0 && KH > 0 && QH % KH == 0 && nbits > 0 && nbits % 32 == 0 && n_max > 0 && k > 0, SL_ERR_SHAPE);
     const int G = QH / KH;
     if (!sl_fused_step_supported(G, nbits / 32, G * nbits + 1, n_max, B, KH)) return 0;
-    const int64_t heads = static_cast<int64_t>(B) * KH;
-    const int64_t b8 = (n_max + 4095) / 4096, b16 = (n_max + 8191) / 8192;
-    if (b8 <= FS_MAX_PEERS && heads * b8 <= sl_fused_step_slots(dtype, G, 4096, !with_lru)) return 1;
-    return b16 <= FS_MAX_PEERS && heads * b16 <= sl_fused_step_slots(dtype, G, 8192, !with_lru) ? 1 : 0;
+    return sl_fused_step_rows(dtype, G, !with_lru, n_max, B, KH) > 0 ? 1 : 0;
 }
 
 extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {

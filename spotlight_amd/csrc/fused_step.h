@@ -3,7 +3,7 @@
 #include "attn.h"
 #include "topk.h"
 
-constexpr int FS_MAX_PEERS = 16;   // blocks of rows (4096 or 8192) per (b, kv head)
+constexpr int FS_MAX_PEERS = 32;   // blocks of rows (1024 ... 8192) per (b, kv head)
 constexpr int FS_NB_PAD = 1028;    // words between the published histograms of two blocks
 
 struct fused_args {
@@ -21,9 +21,9 @@ struct fused_args {
 
 size_t sl_fused_ws_bytes(int B, int KH);
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH);
-// workgroups of the launch the current device holds at once (its grid may not be larger), for the flavour
-// with blocks of `rows` (4096 | 8192) rows, with or without the attention; <= 0: unknown / no such flavour
-int sl_fused_step_slots(int dtype, int G, int rows, bool attend);
+// rows per block the launch would use on the current device for this shape (its workgroups wait for each
+// other, so all of them must be resident at once); 0: the shape cannot take this launch, -1: unknown
+int sl_fused_step_rows(int dtype, int G, bool attend, int64_t n, int B, int KH);
 // sa: n_bins, k, idx, seq_lens (row counts), len_bias, n, B, KH; aa as for sl_attn_launch (aa.idx is ignored).
 // attend false: the launch stops at the list of kept rows (sa.idx); of aa only the shape and the tickets are used.
 int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool attend, void *fused_ws, void *attn_ws,

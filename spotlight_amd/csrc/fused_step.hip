@@ -35,15 +35,18 @@ constexpr int FS_THREADS = FS_NW * 64;
 constexpr int FS_MAX_BPT = 2;                        // histogram bins per lane (<= 1024 bins)
 constexpr uint32_t FS_SPIN_LIMIT = 1u << 22;   // polls a workgroup waits for a peer before it gives up (fused_args::spin_limit)
 
-static_assert(FS_MAX_PEERS == AT_MAX_SPLITS, "one attention run per block of rows");
+static_assert(FS_MAX_PEERS == AT_PART_SPLITS, "one attention run per block of rows");
 
 // FS_SLOTS rows per lane (row = block start + wave * 64 FS_SLOTS + slot * 64 + lane): blocks of 4096
-// rows, or of 8192 where 4096-row blocks would be more workgroups than the device holds at once.
+// rows, of 8192 where 4096-row blocks would be more workgroups than the device holds at once, of 2048
+// or 1024 where a short context keeps many rows (pick_rows).
 // ATTEND false: the launch ends with the list of kept rows (an LRU table update and the attention
 // launch follow); the block that reads its peers' histograms last lowers their flags.
-template <typename T, int G, int FS_SLOTS, bool ATTEND>
+// MAXS: the most blocks a (b, kv head) can have in this launch (16 or 32): the peers' words are loaded all at once.
+template <typename T, int G, int FS_SLOTS, bool ATTEND, int MAXS>
 __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_args fa, select_args sa, attn_args aa) {
     constexpr int W = 4;
+    static_assert(MAXS == 16 || MAXS == 32, "peers polled by the lanes of one wave; merge flavours");
     constexpr int FS_BLOCK = FS_THREADS * FS_SLOTS;
     __shared__ uint32_t s_wave[64];
     __shared__ int s_tn[4];
@@ -160,12 +163,12 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
             const int r = tid * BPT + j;
             cnt[j] = 0u; before[j] = 0u;
             if (j < BPT && r < n_ranks) {   // the loads and their use sit in one block: one round trip for the lanes that have a rank
-                uint32_t raw[FS_MAX_PEERS];
+                uint32_t raw[MAXS];
 #pragma unroll
-                for (int g = 0; g < FS_MAX_PEERS; ++g) raw[g] = ld_agent(peers + (g < S ? g : blk) * FS_NB_PAD + (hi - r));
+                for (int g = 0; g < MAXS; ++g) raw[g] = ld_agent(peers + (g < S ? g : blk) * FS_NB_PAD + (hi - r));
                 uint32_t c = 0, bf = 0;
 #pragma unroll
-                for (int g = 0; g < FS_MAX_PEERS; ++g) {
+                for (int g = 0; g < MAXS; ++g) {
                     const uint32_t v = g < S ? raw[g] : 0u;
                     c += v;
                     bf += g < blk ? v : 0u;
@@ -231,7 +234,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     __syncthreads();
     for (int i = tid; i < n_kept; i += FS_THREADS) out[first + i] = s_list[i];
     if constexpr (ATTEND) {
-        attend_rows_and_merge<T, G, FS_NW>(aa, b, h, blk, S, s_list, n_kept, sh);
+        attend_rows_and_merge<T, G, FS_NW, false, false, MAXS>(aa, b, h, blk, S, s_list, n_kept, sh);
     } else {
         // every lane of this block has used what it read from its peers (the barrier above): the last
         // block of the head to get here lowers the flags for the next launch
@@ -246,7 +249,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     }
 }
 
-int g_fused_rows = 0;  // sl_tune("fused_rows", 0 | 4096 | 8192): rows per block, 0 = 4096 while that fits the device
+int g_fused_rows = 0;  // sl_tune("fused_rows", 0 | 1024 | 2048 | 4096 | 8192): rows per block, 0 = by shape (pick_rows)
 // sl_tune("fused_spin_limit", polls) and sl_tune("fused_phantom_peer", 0 | 1): for the test of the bounded
 // wait -- a short limit and a peer that does not exist make every workgroup give up and report it
 uint32_t g_fused_spin_limit = FS_SPIN_LIMIT;
@@ -254,7 +257,7 @@ int g_fused_phantom_peer = 0;
 
 // workgroups of the kernel the CURRENT device holds at once (looked up once per flavour and device;
 // any thread may ask), 0 when the runtime cannot tell, -1 when the kernel does not fit at all
-template <typename T, int G, int SLOTS, bool ATTEND>
+template <typename T, int G, int SLOTS, bool ATTEND, int MAXS>
 int slots_of() {
     constexpr int MAX_DEV = 64;
     static std::atomic<int> cache[MAX_DEV];   // 0 = not looked up yet
@@ -267,7 +270,7 @@ int slots_of() {
     int per_cu = 0, cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
         hipOccupancyMaxActiveBlocksPerMultiprocessor(
-            &per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G, SLOTS, ATTEND>), FS_THREADS, 0) != hipSuccess) {
+            &per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G, SLOTS, ATTEND, MAXS>), FS_THREADS, 0) != hipSuccess) {
         (void)hipGetLastError();
         return 0;
     }
@@ -276,28 +279,77 @@ int slots_of() {
     return slots;
 }
 
-// Blocks of 4096 rows while all of them fit the device, else of 8192; every workgroup must be able
-// to be resident at once, because workgroups wait for their peers.
+template <typename T, int G, int SLOTS, bool ATTEND, int MAXS>
+int launch_rows(fused_args fa, const select_args &sa, const attn_args &aa, hipStream_t s) {
+    const unsigned heads = static_cast<unsigned>(aa.B) * aa.KH;
+    const int64_t n = sa.n > 0 ? sa.n : 1;
+    fa.blocks = static_cast<unsigned>((n + FS_THREADS * SLOTS - 1) / (FS_THREADS * SLOTS));
+    const dim3 grid(ATTEND ? xcd_grid(heads, fa.blocks) : heads * fa.blocks);
+    score_select_attend_kernel<T, G, SLOTS, ATTEND, MAXS><<<grid, dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
+    return sl_check_launch();
+}
+
+// the flavours that exist: blocks of 4096 and 8192 rows with up to 16 blocks per head; with the attention
+// in the launch also blocks of 1024 and 2048 rows, the latter with up to 16 or up to 32 blocks per head
+template <typename T, int G, bool ATTEND>
+int slots_rows(int rows, bool many) {
+    if (many) {
+        if constexpr (ATTEND) {
+            if (rows == 2048) return slots_of<T, G, 4, true, 32>();
+        }
+        return -1;
+    }
+    switch (rows) {
+        case 8192: return slots_of<T, G, 16, ATTEND, 16>();
+        case 4096: return slots_of<T, G, 8, ATTEND, 16>();
+        case 2048: if constexpr (ATTEND) return slots_of<T, G, 4, true, 16>(); else return -1;
+        case 1024: if constexpr (ATTEND) return slots_of<T, G, 2, true, 16>(); else return -1;
+        default: return -1;
+    }
+}
+
+// Rows per block for a launch over n rows, 0 = the shape cannot take this launch on this device, -1 = the
+// runtime could not tell.  Every workgroup must be resident at once (they wait for their peers).
+// With the attention in the launch: the smallest blocks that give a (b, kv head) at most 16 of them --
+// more, lighter workgroups per head (measured at batch 1, 8k rows: 11.3 us with blocks of 1024 rows
+// against 14.1 with 4096; nine blocks per head is about the optimum).  Where that leaves blocks of 4096
+// rows or more, blocks of 2048 rows with 17 .. 24 per head are taken instead while the whole launch is
+// at most one workgroup per compute unit (batch 1, 32k rows: 14.9 against 15.6 us; at 25 and more
+// blocks, or two workgroups per compute unit, the larger exchange costs more than the lighter blocks save).
+// Without the attention (LRU table): 4096 rows where that fits, else 8192.
+template <typename T, int G, bool ATTEND>
+int pick_rows(int64_t n, int64_t heads) {
+    if (n < 1) n = 1;
+    bool unknown = false;
+    auto fits = [&](int rows, int64_t most_blocks, int64_t most_wgs) {
+        const int64_t blocks = (n + rows - 1) / rows;
+        if (blocks > most_blocks) return false;
+        const int slots = slots_rows<T, G, ATTEND>(rows, blocks > 16);
+        if (slots == 0) unknown = true;
+        return heads * blocks <= (slots < most_wgs ? slots : most_wgs);
+    };
+    constexpr int64_t ANY = int64_t(1) << 40;
+    int rows = 0;
+    if (g_fused_rows) rows = fits(g_fused_rows, FS_MAX_PEERS, ANY) ? g_fused_rows : 0;
+    else if (ATTEND) {
+        rows = fits(1024, 16, ANY) ? 1024 : fits(2048, 16, ANY) ? 2048 : fits(4096, 16, ANY) ? 4096 : fits(8192, 16, ANY) ? 8192 : 0;
+        if (rows >= 4096 && fits(2048, 24, 256)) rows = 2048;
+    } else rows = fits(4096, 16, ANY) ? 4096 : fits(8192, 16, ANY) ? 8192 : 0;
+    return rows == 0 && unknown ? -1 : rows;
+}
+
 template <typename T, int G, bool ATTEND>
 int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, hipStream_t s) {
-    const int64_t heads = static_cast<int64_t>(aa.B) * aa.KH;
-    const int64_t n = sa.n > 0 ? sa.n : 1;
-    const int64_t b8 = (n + 4095) / 4096, b16 = (n + 8191) / 8192;
-    const int s8 = slots_of<T, G, 8, ATTEND>();
-    if (s8 == 0) return SL_ERR_LAUNCH;
-    if (g_fused_rows != 8192 && b8 <= FS_MAX_PEERS && heads * b8 <= s8) {
-        fused_args f8 = fa;
-        f8.blocks = static_cast<unsigned>(b8);
-        score_select_attend_kernel<T, G, 8, ATTEND><<<dim3(ATTEND ? xcd_grid(static_cast<unsigned>(heads), f8.blocks) : static_cast<unsigned>(heads) * f8.blocks), dim3(FS_THREADS), 0, s>>>(f8, sa, aa);
-        return sl_check_launch();
+    const int rows = pick_rows<T, G, ATTEND>(sa.n, static_cast<int64_t>(aa.B) * aa.KH);
+    if (rows < 0) return SL_ERR_LAUNCH;
+    const bool many = ((sa.n > 0 ? sa.n : 1) + rows - 1) / (rows > 0 ? rows : 1) > 16;
+    if constexpr (ATTEND) {
+        if (rows == 2048) return many ? launch_rows<T, G, 4, true, 32>(fa, sa, aa, s) : launch_rows<T, G, 4, true, 16>(fa, sa, aa, s);
+        if (rows == 1024) return many ? SL_ERR_UNSUPPORTED : launch_rows<T, G, 2, true, 16>(fa, sa, aa, s);
     }
-    const int s16 = slots_of<T, G, 16, ATTEND>();
-    if (s16 == 0) return SL_ERR_LAUNCH;
-    SL_REQUIRE(g_fused_rows != 4096 && b16 <= FS_MAX_PEERS && heads * b16 <= s16, SL_ERR_UNSUPPORTED);
-    fused_args f16 = fa;
-    f16.blocks = static_cast<unsigned>(b16);
-    score_select_attend_kernel<T, G, 16, ATTEND><<<dim3(ATTEND ? xcd_grid(static_cast<unsigned>(heads), f16.blocks) : static_cast<unsigned>(heads) * f16.blocks), dim3(FS_THREADS), 0, s>>>(f16, sa, aa);
-    return sl_check_launch();
+    if (rows == 8192) return launch_rows<T, G, 16, ATTEND, 16>(fa, sa, aa, s);
+    if (rows == 4096) return launch_rows<T, G, 8, ATTEND, 16>(fa, sa, aa, s);
+    return SL_ERR_UNSUPPORTED;
 }
 
 template <typename T>
@@ -311,13 +363,12 @@ int launch_t(const fused_args &fa, const select_args &sa, const attn_args &aa, b
 }
 
 template <typename T>
-int slots_t(int G, int rows, bool attend) {
-    const bool big = rows == 8192;
+int pick_t(int G, bool attend, int64_t n, int64_t heads) {
     switch (G) {
-        case 1: return attend ? (big ? slots_of<T, 1, 16, true>() : slots_of<T, 1, 8, true>()) : (big ? slots_of<T, 1, 16, false>() : slots_of<T, 1, 8, false>());
-        case 2: return attend ? (big ? slots_of<T, 2, 16, true>() : slots_of<T, 2, 8, true>()) : (big ? slots_of<T, 2, 16, false>() : slots_of<T, 2, 8, false>());
-        case 4: return attend ? (big ? slots_of<T, 4, 16, true>() : slots_of<T, 4, 8, true>()) : (big ? slots_of<T, 4, 16, false>() : slots_of<T, 4, 8, false>());
-        default: return -1;
+        case 1: return attend ? pick_rows<T, 1, true>(n, heads) : pick_rows<T, 1, false>(n, heads);
+        case 2: return attend ? pick_rows<T, 2, true>(n, heads) : pick_rows<T, 2, false>(n, heads);
+        case 4: return attend ? pick_rows<T, 4, true>(n, heads) : pick_rows<T, 4, false>(n, heads);
+        default: return 0;
     }
 }
 
@@ -330,25 +381,25 @@ size_t sl_fused_ws_bytes(int B, int KH) {
 }
 
 int sl_fused_tune(const char *key, int value) {
-    if (!strcmp(key, "fused_rows") && (value == 0 || value == 4096 || value == 8192)) { g_fused_rows = value; return SL_OK; }
+    if (!strcmp(key, "fused_rows") && (value == 0 || value == 1024 || value == 2048 || value == 4096 || value == 8192)) { g_fused_rows = value; return SL_OK; }
     if (!strcmp(key, "fused_spin_limit") && value >= 0) { g_fused_spin_limit = value ? static_cast<uint32_t>(value) : FS_SPIN_LIMIT; return SL_OK; }
     if (!strcmp(key, "fused_phantom_peer") && (value == 0 || value == 1)) { g_fused_phantom_peer = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
 
-int sl_fused_step_slots(int dtype, int G, int rows, bool attend) {
-    if (rows != 4096 && rows != 8192) return -1;
+int sl_fused_step_rows(int dtype, int G, bool attend, int64_t n, int B, int KH) {
+    const int64_t heads = static_cast<int64_t>(B) * KH;
     switch (dtype) {
-        case SL_F32: return slots_t<float>(G, rows, attend);
-        case SL_BF16: return slots_t<bf16_t>(G, rows, attend);
-        case SL_F16: return slots_t<f16_t>(G, rows, attend);
-        default: return -1;
+        case SL_F32: return pick_t<float>(G, attend, n, heads);
+        case SL_BF16: return pick_t<bf16_t>(G, attend, n, heads);
+        case SL_F16: return pick_t<f16_t>(G, attend, n, heads);
+        default: return 0;
     }
 }
 
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH) {
     return (G == 1 || G == 2 || G == 4) && W == 4 && n_bins <= FS_THREADS * FS_MAX_BPT && n_bins <= FS_NB_PAD &&
-           (n + 8191) / 8192 <= FS_MAX_PEERS && B <= 65535 && KH <= 65535;
+           (n + 8191) / 8192 <= 16 && B <= 65535 && KH <= 65535;
 }
 
 int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool attend, void *fused_ws, void *attn_ws,
@@ -367,7 +418,7 @@ int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool atten
     aa.peer_flag = fa.peer_flag;
     fa.spin_limit = g_fused_spin_limit;
     // (a phantom needs a free flag slot: heads that already have 16 blocks get none)
-    fa.phantom_peers = g_fused_phantom_peer && (sa.n + 4095) / 4096 < FS_MAX_PEERS ? 1 : 0;
+    fa.phantom_peers = g_fused_phantom_peer && (sa.n + 1023) / 1024 < 16 ? 1 : 0;   // (stays within the 16-block flavours)
     switch (aa.dtype) {
         case SL_F32: return launch_t<float>(fa, sa, aa, attend, s);
         case SL_BF16: return launch_t<bf16_t>(fa, sa, aa, attend, s);

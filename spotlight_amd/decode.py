@@ -98,14 +98,15 @@ class LayerDecodeState:
         # takes head-major whenever that launch covers the shape.  ``codes`` is always indexed
         # [b, row, kv head, word]; with head-major storage it is a strided view.
         if codes_layout == "auto":
-            # without an LRU table the launch also attends, one run per block: keep <= 128 rows per 4096
-            # (and stay with the three launches beyond 64k rows: measured no faster there)
-            rows_ok = bool(lru_slots) or (k <= 128 * ((n_cap + 4095) // 4096) and n_cap <= 65536)
+            # without an LRU table the launch also attends, one run per block of rows (9 to 24 blocks of
+            # 1024 ... 8192 rows): keep <= 128 rows per block on average (and stay with the three launches
+            # beyond 64k rows: measured no faster there)
+            rows_ok = bool(lru_slots) or (k <= 128 * min(16, (n_cap + 1023) // 1024) and n_cap <= 65536)
             fits = 0
             if rows_ok and W == 4:
                 # all blocks of a launch must be resident at once; the library knows what the device holds
                 with torch.cuda.device(dev):
-                    fits = _lib.load().sl_decode_head_major_fits(K._DTYPES[self.dtype], B, QH, KH, self.nbits, n_cap,
+                    fits = _lib.load().sl_decode_head_major_fits(K._DTYPES[self.dtype], B, QH, KH, self.nbits, n_cap, k,
                                                                  int(bool(lru_slots)))
             codes_layout = "head" if fits > 0 else "token"
         assert codes_layout in ("token", "head")

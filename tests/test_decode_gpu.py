@@ -321,7 +321,7 @@ def test_decode_many_blocks_and_long_cache(env):
     two-launch selector once the copies wrap around (beyond 256k tokens)."""
     decode, kernel = env
     for n0, k, layout in ((9000, 180, "token"), (9000, 180, "head"), (20000, 100, "token"), (20000, 100, "head"),
-                          (60000, 300, "head"), (70000, 300, "auto"), (140000, 500, "auto"), (270000, 64, "auto")):
+                          (40000, 200, "head"), (60000, 300, "head"), (70000, 300, "auto"), (140000, 500, "auto"), (270000, 64, "auto")):
         g = _gen(n0)
         st = _make_state(decode, g, 1, 8, 2, n0, (n0 + 64 + 7) // 8 * 8, k, torch.bfloat16, codes_layout=layout)
         assert st.codes_layout == ("token" if n0 > 65000 else layout if layout != "auto" else "head")
@@ -333,10 +333,9 @@ def test_decode_many_blocks_and_long_cache(env):
             _check_step(kernel, st, q, kn, vn, out, n0 + step, torch.bfloat16)
 
 
-@pytest.mark.parametrize("rows", [4096, 8192])
-@pytest.mark.parametrize("lru", [0, 512])
-def test_head_major_blocks_of_4096_and_8192_rows(env, rows, lru):
-    """Head-major codes with several blocks per (b, kv head), in both block sizes, without and with
+@pytest.mark.parametrize("rows,lru", [(4096, 0), (8192, 0), (4096, 512), (8192, 512), (1024, 0), (2048, 0)])
+def test_head_major_blocks_of_every_size(env, rows, lru):
+    """Head-major codes with several blocks per (b, kv head), in every block size, without and with
     the LRU table (where the launch ends at the selection and lowers its own flags): every step
     equals the oracle and the state with token-major codes, over a block boundary."""
     decode, kernel = env
@@ -371,8 +370,7 @@ def test_head_major_blocks_of_4096_and_8192_rows(env, rows, lru):
         _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
 
 
-@pytest.mark.parametrize("lru", [0, 256])
-@pytest.mark.parametrize("rows", [4096, 8192])
+@pytest.mark.parametrize("rows,lru", [(4096, 0), (8192, 0), (4096, 256), (8192, 256), (1024, 0), (2048, 0)])
 def test_head_major_ragged_batch_with_different_block_counts(env, rows, lru):
     """One batch whose sequences have 1, 2 and 3 blocks of rows (and one that ends exactly on a block
     boundary, so the step opens a new block): every (b, kv head) swaps histograms among ITS blocks
@@ -427,7 +425,9 @@ def test_head_major_equals_token_major_on_random_shapes(env):
             k = rnd.choice([1, 7, 64, 100, 300, 600])
             lru = rnd.choice([0, 0, 1024])
             dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
-            rows = rnd.choice([0, 4096, 8192])
+            rows = rnd.choice([0, 4096, 8192, 1024, 2048])
+            if rows in (1024, 2048) and (lru or n0 + 3 > 16 * rows):   # the small blocks: attention in the launch, <= 16 blocks
+                rows = 0
             n_cap = (n0 + 16 + 7) // 8 * 8
             cg = torch.Generator().manual_seed(case)
             g = torch.Generator(device=DEV).manual_seed(case)
