@@ -3,7 +3,7 @@
 #include "attn.h"
 #include "topk.h"
 
-constexpr int FS_MAX_PEERS = 32;   // blocks of rows (1024 ... 8192) per (b, kv head)
+constexpr int FS_MAX_PEERS = 16;   // blocks of rows (512 ... 8192) per (b, kv head)
 constexpr int FS_NB_PAD = 1028;    // words between the published histograms of two blocks
 
 struct fused_args {
@@ -29,3 +29,13 @@ int sl_fused_step_rows(int dtype, int G, bool attend, int64_t n, int B, int KH);
 int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool attend, void *fused_ws, void *attn_ws,
                          size_t attn_ws_bytes, hipStream_t s);
 int sl_fused_tune(const char *key, int value);
+
+// per element type (fused_step_<type>.hip)
+int sl_fused_launch_f32(const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s);
+int sl_fused_launch_bf16(const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s);
+int sl_fused_launch_f16(const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s);
+int sl_fused_pick_f32(int G, bool attend, int64_t n, int64_t heads);
+int sl_fused_pick_bf16(int G, bool attend, int64_t n, int64_t heads);
+int sl_fused_pick_f16(int G, bool attend, int64_t n, int64_t heads);
+extern int g_fused_rows;                       // sl_tune("fused_rows")
+constexpr uint32_t FS_SPIN_LIMIT = 1u << 22;   // polls a workgroup waits for a peer before it gives up (fused_args::spin_limit)

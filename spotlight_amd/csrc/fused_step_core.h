@@ -1,0 +1,363 @@
+// Kernel and launch templates of the one-launch scorer + selection + attention over head-major codes
+// (what fused_step.hip describes), instantiated per element type in fused_step_<type>.hip.
+#pragma once
+#include "fused_step.h"
+
+#include <atomic>
+
+#include "attn_core.h"
+#include "topk_core.h"
+
+namespace {
+
+
+constexpr int FS_NW = 8;
+constexpr int FS_THREADS = FS_NW * 64;
+constexpr int FS_MAX_BPT = 2;                        // histogram bins per lane (<= 1024 bins: sl_fused_step_supported)
+
+static_assert(FS_MAX_PEERS == AT_MAX_SPLITS, "one attention run per block of rows");
+
+// FS_SLOTS rows per lane (row = block start + wave * 64 FS_SLOTS + slot * 64 + lane): blocks of
+// 512 FS_SLOTS rows; pick_rows chooses the size by shape.
+// ATTEND false: the launch ends with the list of kept rows (an LRU table update and the attention
+// launch follow); the block that reads its peers' histograms last lowers their flags.
+// MAXS: the most blocks a (b, kv head) can have in this launch: the peers' words are loaded all at once.
+template <typename T, int G, int FS_SLOTS, bool ATTEND, int MAXS>
+__global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_args fa, select_args sa, attn_args aa) {
+    constexpr int W = 4;
+    static_assert(MAXS == 16, "peers polled by the lanes of one wave; merge flavour");
+    constexpr int FS_BLOCK = FS_THREADS * FS_SLOTS;
+    __shared__ uint32_t s_wave[64];
+    __shared__ int s_tn[4];
+    __shared__ uint32_t s_hist[FS_THREADS * FS_MAX_BPT];
+    __shared__ uint32_t s_cnt[FS_NW];
+    __shared__ int s_range[2];
+    __shared__ int32_t s_list[FS_BLOCK];
+    __shared__ attn_shared<ATTEND ? G : 1, FS_NW> sh;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // With the attention in the launch the blocks of a (b, kv head) share an XCD (see xcd_unmap): they swap
+    // histograms and merge their runs (measured: 0.5 - 0.7 us per step at batch 1 - 3).  Without it, and for
+    // the attention and select + attend launches, neighbouring numbering measured as fast or faster.
+    int bh, blk;
+    if constexpr (ATTEND) {
+        if (!xcd_unmap(blockIdx.x, static_cast<unsigned>(aa.B) * sa.KH, fa.blocks, bh, blk)) return;
+    } else {
+        bh = static_cast<int>(blockIdx.x / fa.blocks);
+        blk = static_cast<int>(blockIdx.x % fa.blocks);
+    }
+    const int b = bh / sa.KH, h = bh % sa.KH;
+    const int NB = sa.n_bins;
+
+    // loads first: the G query codes of this kv head and the lane's 8 rows; none needs the row count
+    // (rows past the bound fa.n re-read the last row and are discarded below)
+    const uint32_t *qb = fa.q_code + static_cast<int64_t>(b) * fa.q_stride_b;
+    uint4 qreg[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int qh = fa.head_map == SL_HEADMAP_BLOCKED ? h * G + g : g * sa.KH + h;
+        qreg[g] = *reinterpret_cast<const uint4 *>(qb + static_cast<int64_t>(qh) * W);
+    }
+    const uint4 *kb = reinterpret_cast<const uint4 *>(fa.k_code + static_cast<int64_t>(b) * fa.k_stride_b +
+                                                      static_cast<int64_t>(h) * fa.k_stride_h);
+    const int64_t t_base = static_cast<int64_t>(blk) * FS_BLOCK + wave * (64 * FS_SLOTS) + lane;
+    uint4 kreg[FS_SLOTS];
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        const int64_t t = t_base + j * 64;
+        kreg[j] = kb[t < sa.n ? t : sa.n - 1];
+    }
+    const int64_t n_b = tokens_of(sa, b);
+    const int k_eff = n_b < sa.k ? static_cast<int>(n_b) : sa.k;
+    int32_t *out = sa.idx + static_cast<int64_t>(bh) * sa.k;
+    if (blk == 0)
+        for (int i = k_eff + tid; i < sa.k; i += FS_THREADS) out[i] = -1;
+    if (static_cast<int64_t>(blk) * FS_BLOCK >= n_b) return;
+    const int S = static_cast<int>((n_b + FS_BLOCK - 1) / FS_BLOCK);  // blocks (= attention runs) of this (b, kv head)
+
+    for (int e = tid; e < FS_THREADS * FS_MAX_BPT; e += FS_THREADS) s_hist[e] = 0;
+    if (tid == 0) { s_range[0] = NB; s_range[1] = -1; }
+    __syncthreads();
+
+    // scores: matching bits summed over the G query heads; -1 marks a row past the end
+    int sc[FS_SLOTS];
+    int s_lo = NB, s_hi = -1;
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        int dist = 0;
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+            dist += __popc(qreg[g].x ^ kreg[j].x) + __popc(qreg[g].y ^ kreg[j].y) + __popc(qreg[g].z ^ kreg[j].z) +
+                    __popc(qreg[g].w ^ kreg[j].w);
+        const bool valid = t_base + j * 64 < n_b;
+        sc[j] = valid ? G * W * 32 - dist : -1;
+        if (valid) {
+            atomicAdd(&s_hist[sc[j]], 1u);
+            s_lo = sc[j] < s_lo ? sc[j] : s_lo;
+            s_hi = sc[j] > s_hi ? sc[j] : s_hi;
+        }
+    }
+    // the block's score range: only these bins of its histogram can be non-empty
+    s_lo = wave_min_i32(s_lo);
+    s_hi = wave_max_i32(s_hi);
+    if (lane == 0) { atomicMin(&s_range[0], s_lo); atomicMax(&s_range[1], s_hi); }
+    __syncthreads();
+
+    // Histogram of the whole (b, kv head), restricted to [lo, hi], the union of the blocks' score ranges:
+    // bin hi - r is rank r.  cnt = this lane's ranks summed over the blocks, before = over the blocks in
+    // front of this one.
+    int lo = s_range[0], hi = s_range[1];   // a block that got here holds at least one row: lo <= hi
+    uint32_t cnt[FS_MAX_BPT], before[FS_MAX_BPT], mine = 0;
+    if (S > 1) {
+        uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * FS_MAX_PEERS * FS_NB_PAD;
+        uint32_t *flags = fa.peer_flag + static_cast<int64_t>(bh) * FS_MAX_PEERS;
+        // every bin is published, zeros included: the peers read the union of all ranges
+        for (int e = tid; e < NB; e += FS_THREADS) st_agent(peers + blk * FS_NB_PAD + e, s_hist[e]);
+        publish_wait();
+        __syncthreads();
+        // the flag carries the block's range: bit 31 = published, bits 12.. = hi, bits 0..11 = lo
+        if (tid == 0) st_agent(flags + blk, 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo));
+        if (wave == 0) {
+            uint32_t f = 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo);
+            if (lane < S + fa.phantom_peers) {   // (phantom_peers: a flag nobody raises, to exercise the bounded wait)
+                uint32_t spins = 0;
+                while (((f = ld_agent(flags + lane)) & 0x80000000u) == 0u) {
+                    if (++spins > fa.spin_limit) { st_agent(fa.error, 1u); f = 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo); break; }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            const int all_lo = wave_min_i32(static_cast<int>(f & 0xfffu));
+            const int all_hi = wave_max_i32(static_cast<int>((f >> 12) & 0xfffu));
+            if (lane == 0) { s_range[0] = all_lo; s_range[1] = all_hi; }
+        }
+        __syncthreads();
+        lo = s_range[0]; hi = s_range[1];
+    }
+    const int n_ranks = hi - lo + 1;
+    const int BPT = (n_ranks + FS_THREADS - 1) / FS_THREADS;
+    if (S > 1) {
+        const uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * FS_MAX_PEERS * FS_NB_PAD;
+#pragma unroll
+        for (int j = 0; j < FS_MAX_BPT; ++j) {
+            const int r = tid * BPT + j;
+            cnt[j] = 0u; before[j] = 0u;
+            if (j < BPT && r < n_ranks) {   // the loads and their use sit in one block: one round trip for the lanes that have a rank
+                uint32_t raw[MAXS];
+#pragma unroll
+                for (int g = 0; g < MAXS; ++g) raw[g] = ld_agent(peers + (g < S ? g : blk) * FS_NB_PAD + (hi - r));
+                uint32_t c = 0, bf = 0;
+#pragma unroll
+                for (int g = 0; g < MAXS; ++g) {
+                    const uint32_t v = g < S ? raw[g] : 0u;
+                    c += v;
+                    bf += g < blk ? v : 0u;
+                }
+                cnt[j] = c; before[j] = bf;
+            }
+            mine += cnt[j];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < FS_MAX_BPT; ++j) {
+            const int r = tid * BPT + j;
+            cnt[j] = (j < BPT && r < n_ranks) ? s_hist[hi - r] : 0u;
+            before[j] = 0u;
+            mine += cnt[j];
+        }
+    }
+
+    int thr, need;
+    uint32_t tg, te;
+    find_threshold<FS_THREADS, FS_MAX_BPT>(hi, n_ranks, cnt, before, mine, k_eff, s_wave, s_tn, thr, need, tg, te);
+
+    // placement in row order (wave, slot, lane): ballots give every kept row its position
+    uint32_t mgt_lo[FS_SLOTS], mgt_hi[FS_SLOTS], meq_lo[FS_SLOTS], meq_hi[FS_SLOTS];
+    uint32_t wave_gt = 0, wave_eq = 0;
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        const uint64_t mg = __ballot(sc[j] > thr), me = __ballot(sc[j] == thr);
+        mgt_lo[j] = static_cast<uint32_t>(mg); mgt_hi[j] = static_cast<uint32_t>(mg >> 32);
+        meq_lo[j] = static_cast<uint32_t>(me); meq_hi[j] = static_cast<uint32_t>(me >> 32);
+        wave_gt += __popc(mgt_lo[j]) + __popc(mgt_hi[j]);
+        wave_eq += __popc(meq_lo[j]) + __popc(meq_hi[j]);
+    }
+    if (lane == 0) s_cnt[wave] = wave_gt | (wave_eq << 16);
+    __syncthreads();
+    uint32_t gt_before = tg, eq_before = te, tot_gt = 0, tot_eq = 0;
+#pragma unroll
+    for (int w = 0; w < FS_NW; ++w) {
+        const uint32_t c = s_cnt[w];
+        tot_gt += c & 0xffffu; tot_eq += c >> 16;
+        gt_before += w < wave ? (c & 0xffffu) : 0u;
+        eq_before += w < wave ? (c >> 16) : 0u;
+    }
+    const uint32_t uneed = static_cast<uint32_t>(need);
+    const uint32_t first = tg + (te < uneed ? te : uneed);   // output position of the block's first kept row
+#pragma unroll
+    for (int j = 0; j < FS_SLOTS; ++j) {
+        const uint32_t g_here = gt_before + __builtin_amdgcn_mbcnt_hi(mgt_hi[j], __builtin_amdgcn_mbcnt_lo(mgt_lo[j], 0u));
+        const uint32_t e_here = eq_before + __builtin_amdgcn_mbcnt_hi(meq_hi[j], __builtin_amdgcn_mbcnt_lo(meq_lo[j], 0u));
+        const bool above = sc[j] > thr, equal = sc[j] == thr;
+        const uint32_t pos = g_here + (e_here < uneed ? e_here : uneed);
+        if ((above || (equal && e_here < uneed)) && pos < static_cast<uint32_t>(k_eff))
+            s_list[pos - first] = static_cast<int32_t>(t_base + j * 64);
+        gt_before += __popc(mgt_lo[j]) + __popc(mgt_hi[j]);
+        eq_before += __popc(meq_lo[j]) + __popc(meq_hi[j]);
+    }
+    const uint32_t eq_end = te + tot_eq;
+    uint32_t end = tg + tot_gt + (eq_end < uneed ? eq_end : uneed);
+    if (end > static_cast<uint32_t>(k_eff)) end = static_cast<uint32_t>(k_eff);
+    const int n_kept = end > first ? static_cast<int>(end - first) : 0;
+
+    // the list goes out with coalesced stores; the attention then runs over it
+    __syncthreads();
+    for (int i = tid; i < n_kept; i += FS_THREADS) out[first + i] = s_list[i];
+    if constexpr (ATTEND) {
+        attend_rows_and_merge<T, G, FS_NW, false, false, MAXS>(aa, b, h, blk, S, s_list, n_kept, sh);
+    } else {
+        // every lane of this block has used what it read from its peers (the barrier above): the last
+        // block of the head to get here lowers the flags for the next launch
+        if (S > 1 && wave == 0) {
+            uint32_t last = 0;
+            if (lane == 0) last = arrive_last(&aa.counter[bh], static_cast<uint32_t>(S)) ? 1u : 0u;
+            if (__builtin_amdgcn_readfirstlane(last)) {
+                if (lane < S) st_agent(fa.peer_flag + static_cast<int64_t>(bh) * FS_MAX_PEERS + lane, 0u);
+                if (lane == 0) st_agent(&aa.counter[bh], 0u);
+            }
+        }
+    }
+}
+
+// workgroups of the kernel the CURRENT device holds at once (looked up once per flavour and device;
+// any thread may ask), 0 when the runtime cannot tell, -1 when the kernel does not fit at all
+template <typename T, int G, int SLOTS, bool ATTEND, int MAXS>
+int slots_of() {
+    constexpr int MAX_DEV = 64;
+    static std::atomic<int> cache[MAX_DEV];   // 0 = not looked up yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    if (dev >= 0 && dev < MAX_DEV) {
+        const int known = cache[dev].load(std::memory_order_relaxed);
+        if (known != 0) return known;
+    }
+    int per_cu = 0, cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &per_cu, reinterpret_cast<const void *>(&score_select_attend_kernel<T, G, SLOTS, ATTEND, MAXS>), FS_THREADS, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    const int slots = per_cu * cus > 0 ? per_cu * cus : -1;
+    if (dev >= 0 && dev < MAX_DEV) cache[dev].store(slots, std::memory_order_relaxed);
+    return slots;
+}
+
+template <typename T, int G, int SLOTS, bool ATTEND, int MAXS>
+int launch_rows(fused_args fa, const select_args &sa, const attn_args &aa, hipStream_t s) {
+    const unsigned heads = static_cast<unsigned>(aa.B) * aa.KH;
+    const int64_t n = sa.n > 0 ? sa.n : 1;
+    fa.blocks = static_cast<unsigned>((n + FS_THREADS * SLOTS - 1) / (FS_THREADS * SLOTS));
+    if (fa.blocks >= FS_MAX_PEERS) fa.phantom_peers = 0;   // a phantom peer needs a free flag
+    const dim3 grid(ATTEND ? xcd_grid(heads, fa.blocks) : heads * fa.blocks);
+    score_select_attend_kernel<T, G, SLOTS, ATTEND, MAXS><<<grid, dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
+    return sl_check_launch();
+}
+
+// Rows per block come in multiples of 512 (one row per lane): the flavours that exist.
+constexpr int FS_FLAVOURS[] = {1, 2, 3, 4, 5, 6, 7, 8, 16};
+
+template <typename T, int G, bool ATTEND>
+int slots_rows(int slots_per_lane) {
+    switch (slots_per_lane) {
+        case 16: return slots_of<T, G, 16, ATTEND, 16>();
+        case 8: return slots_of<T, G, 8, ATTEND, 16>();
+        default: break;
+    }
+    if constexpr (ATTEND) {
+        switch (slots_per_lane) {
+            case 1: return slots_of<T, G, 1, true, 16>();
+            case 2: return slots_of<T, G, 2, true, 16>();
+            case 3: return slots_of<T, G, 3, true, 16>();
+            case 4: return slots_of<T, G, 4, true, 16>();
+            case 5: return slots_of<T, G, 5, true, 16>();
+            case 6: return slots_of<T, G, 6, true, 16>();
+            case 7: return slots_of<T, G, 7, true, 16>();
+            default: break;
+        }
+    }
+    return -1;
+}
+
+// Rows per block for a launch over n rows, 0 = the shape cannot take this launch on this device, -1 = the
+// runtime could not tell.  Every workgroup must be resident at once (they wait for their peers) and a
+// (b, kv head) has at most 16 blocks.  With the attention in the launch: the smallest blocks that
+// satisfy both -- more, lighter workgroups per head (measured at batch 1: 8k rows, 9 blocks of 1024:
+// 11.3 us against 14.1 with 2 of 4096; 32k rows, 13 blocks of 2560: 14.1 against 15.5 with 9 of 4096;
+// 40k rows, 16 of 2560: 14.7 against 16.0 with 10 of 4096; more than 16 blocks measured slower again,
+// and so did more than 8 rows per lane).  Without the attention (LRU table): 4096 rows where that
+// fits, else 8192.
+template <typename T, int G, bool ATTEND>
+int pick_rows(int64_t n, int64_t heads) {
+    if (n < 1) n = 1;
+    bool unknown = false;
+    auto fits = [&](int spl) {
+        const int64_t rows = 512 * spl, blocks = (n + rows - 1) / rows;
+        if (blocks > FS_MAX_PEERS) return false;
+        const int slots = slots_rows<T, G, ATTEND>(spl);
+        if (slots == 0) unknown = true;
+        return heads * blocks <= slots;
+    };
+    int spl = 0;
+    if (g_fused_rows) spl = g_fused_rows % 512 == 0 && fits(g_fused_rows / 512) ? g_fused_rows / 512 : 0;
+    else if (ATTEND) {
+        for (int f : FS_FLAVOURS)
+            if (spl == 0 && fits(f)) spl = f;
+    } else spl = fits(8) ? 8 : fits(16) ? 16 : 0;
+    return spl == 0 && unknown ? -1 : 512 * spl;
+}
+
+template <typename T, int G, bool ATTEND>
+int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, hipStream_t s) {
+    const int rows = pick_rows<T, G, ATTEND>(sa.n, static_cast<int64_t>(aa.B) * aa.KH);
+    if (rows < 0) return SL_ERR_LAUNCH;
+    switch (rows / 512) {
+        case 16: return launch_rows<T, G, 16, ATTEND, 16>(fa, sa, aa, s);
+        case 8: return launch_rows<T, G, 8, ATTEND, 16>(fa, sa, aa, s);
+        default: break;
+    }
+    if constexpr (ATTEND) {
+        switch (rows / 512) {
+            case 1: return launch_rows<T, G, 1, true, 16>(fa, sa, aa, s);
+            case 2: return launch_rows<T, G, 2, true, 16>(fa, sa, aa, s);
+            case 3: return launch_rows<T, G, 3, true, 16>(fa, sa, aa, s);
+            case 4: return launch_rows<T, G, 4, true, 16>(fa, sa, aa, s);
+            case 5: return launch_rows<T, G, 5, true, 16>(fa, sa, aa, s);
+            case 6: return launch_rows<T, G, 6, true, 16>(fa, sa, aa, s);
+            case 7: return launch_rows<T, G, 7, true, 16>(fa, sa, aa, s);
+            default: break;
+        }
+    }
+    return SL_ERR_UNSUPPORTED;
+}
+
+template <typename T>
+int fused_launch_t(const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s) {
+    switch (aa.QH / aa.KH) {
+        case 1: return attend ? launch_tg<T, 1, true>(fa, sa, aa, s) : launch_tg<T, 1, false>(fa, sa, aa, s);
+        case 2: return attend ? launch_tg<T, 2, true>(fa, sa, aa, s) : launch_tg<T, 2, false>(fa, sa, aa, s);
+        case 4: return attend ? launch_tg<T, 4, true>(fa, sa, aa, s) : launch_tg<T, 4, false>(fa, sa, aa, s);
+        default: return SL_ERR_UNSUPPORTED;
+    }
+}
+
+template <typename T>
+int fused_pick_t(int G, bool attend, int64_t n, int64_t heads) {
+    switch (G) {
+        case 1: return attend ? pick_rows<T, 1, true>(n, heads) : pick_rows<T, 1, false>(n, heads);
+        case 2: return attend ? pick_rows<T, 2, true>(n, heads) : pick_rows<T, 2, false>(n, heads);
+        case 4: return attend ? pick_rows<T, 4, true>(n, heads) : pick_rows<T, 4, false>(n, heads);
+        default: return 0;
+    }
+}
+
+}  // namespace
