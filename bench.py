@@ -570,8 +570,10 @@ def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False):
     grids = [((QH + KH) * ((B + hash_rows - 1) // hash_rows), 512),
              (((n_max * KH + 2047) // 2048) * B, 512)]
     if one_launch_tail:
-        # blocks of 4096 rows while the device holds them all at once (two 8-wave workgroups per compute unit), else 8192
-        blocks = blocks4k if blocks4k * KH * B <= 512 else (n_max + 8191) // 8192
+        # the library picks the rows per block by shape and by what the device holds at once
+        dt = {"f32": 0, "bf16": 1, "f16": 2}[c["dtype"]]
+        rows = lib.sl_decode_head_major_fits(dt, B, QH, KH, 128, n_max, c["k"], int(bool(c["lru"])))
+        blocks = (n_max + rows - 1) // rows if rows > 0 else blocks4k
         grids = [grids[0], (blocks * KH * B, 512)]
         if c["lru"]:
             grids += [(B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]

@@ -319,12 +319,13 @@ size_t sl_decode_workspace_bytes(const sl_decode_params *p);
  * blocks of its (b, kv head) (results of that step are then wrong); (size_t)-1 when
  * the parameters do not use that launch.  It stays 0 in a healthy run. */
 size_t sl_decode_error_offset(const sl_decode_params *p);
-/* 1 if sl_decode_step can run this shape over head-major codes on the current
- * device, 0 if not (the caller then keeps token-major codes), negative on bad
- * arguments.  The blocks of rows of such a launch (4096 rows; 8192 when that is
- * what fits; 2048 or 1024 when a short context keeps many rows) wait for each other, so B * KH * blocks may not exceed the workgroups
- * the device holds at once; n_max is the largest row bound the caller will pass
- * (its n_cap).  No counterpart in the reference. */
+/* Whether sl_decode_step can run this shape over head-major codes on the current
+ * device: the rows per block it would use (> 0), 0 if it cannot (the caller then
+ * keeps token-major codes), negative on bad arguments.  The blocks of rows of such a
+ * launch (512 to 8192 rows: the smallest that give a (b, kv head) at most 16 blocks)
+ * wait for each other, so B * KH * blocks may not exceed the workgroups the device
+ * holds at once; n_max is the largest row bound the caller will pass (its n_cap).
+ * No counterpart in the reference. */
 int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int k, int with_lru);
 int sl_decode_step(const sl_decode_params *p, void *stream);
 

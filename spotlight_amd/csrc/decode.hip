@@ -151,7 +151,8 @@ extern "C" int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int n
     SL_REQUIRE(B > 0 && QH > 0 && KH > 0 && QH % KH == 0 && nbits > 0 && nbits % 32 == 0 && n_max > 0 && k > 0, SL_ERR_SHAPE);
     const int G = QH / KH;
     if (!sl_fused_step_supported(G, nbits / 32, G * nbits + 1, n_max, B, KH)) return 0;
-    return sl_fused_step_rows(dtype, G, !with_lru, n_max, B, KH) > 0 ? 1 : 0;
+    const int rows = sl_fused_step_rows(dtype, G, !with_lru, n_max, B, KH);
+    return rows > 0 ? rows : 0;
 }
 
 extern "C" int sl_decode_step(const sl_decode_params *pp, void *stream) {
