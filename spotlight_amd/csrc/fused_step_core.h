@@ -264,7 +264,7 @@ int launch_rows(fused_args fa, const select_args &sa, const attn_args &aa, hipSt
 }
 
 // Rows per block come in multiples of 512 (one row per lane): the flavours that exist.
-constexpr int FS_FLAVOURS[] = {1, 2, 3, 4, 5, 6, 7, 8, 16};
+constexpr int FS_FLAVOURS[] = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 14, 16};
 
 template <typename T, int G, bool ATTEND>
 int slots_rows(int slots_per_lane) {
@@ -282,6 +282,11 @@ int slots_rows(int slots_per_lane) {
             case 5: return slots_of<T, G, 5, true, 16>();
             case 6: return slots_of<T, G, 6, true, 16>();
             case 7: return slots_of<T, G, 7, true, 16>();
+            case 9: return slots_of<T, G, 9, true, 16>();
+            case 10: return slots_of<T, G, 10, true, 16>();
+            case 11: return slots_of<T, G, 11, true, 16>();
+            case 12: return slots_of<T, G, 12, true, 16>();
+            case 14: return slots_of<T, G, 14, true, 16>();
             default: break;
         }
     }
@@ -294,8 +299,9 @@ int slots_rows(int slots_per_lane) {
 // satisfy both -- more, lighter workgroups per head (measured at batch 1: 8k rows, 9 blocks of 1024:
 // 11.3 us against 14.1 with 2 of 4096; 32k rows, 13 blocks of 2560: 14.1 against 15.5 with 9 of 4096;
 // 40k rows, 16 of 2560: 14.7 against 16.0 with 10 of 4096; more than 16 blocks measured slower again,
-// and so did more than 8 rows per lane).  Without the attention (LRU table): 4096 rows where that
-// fits, else 8192.
+// and so did more than 8 rows per lane, which therefore only come in where fewer, larger blocks are
+// what it takes to keep the grid resident: batch 8 at 32k rows).  Without the attention (LRU table):
+// 4096 rows where that fits, else 8192.
 template <typename T, int G, bool ATTEND>
 int pick_rows(int64_t n, int64_t heads) {
     if (n < 1) n = 1;
@@ -334,6 +340,11 @@ int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, 
             case 5: return launch_rows<T, G, 5, true, 16>(fa, sa, aa, s);
             case 6: return launch_rows<T, G, 6, true, 16>(fa, sa, aa, s);
             case 7: return launch_rows<T, G, 7, true, 16>(fa, sa, aa, s);
+            case 9: return launch_rows<T, G, 9, true, 16>(fa, sa, aa, s);
+            case 10: return launch_rows<T, G, 10, true, 16>(fa, sa, aa, s);
+            case 11: return launch_rows<T, G, 11, true, 16>(fa, sa, aa, s);
+            case 12: return launch_rows<T, G, 12, true, 16>(fa, sa, aa, s);
+            case 14: return launch_rows<T, G, 14, true, 16>(fa, sa, aa, s);
             default: break;
         }
     }
