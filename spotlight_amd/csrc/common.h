@@ -201,6 +201,16 @@ __device__ __forceinline__ void st_agent(uint32_t *p, uint32_t v) {
 __device__ __forceinline__ uint32_t ld_agent(const uint32_t *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// compute units of the current device (0: the runtime could not tell)
+inline int sl_compute_units() {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return cus;
+}
+
 // Workgroups of a 1-D grid go to the device's 8 XCDs (each with its own L2) in turn: workgroup i
 // runs on XCD (i + c) % 8.  Work items that exchange data -- the parts of one group -- are therefore
 // numbered so that a group's parts share i % 8: their device-coherent stores and loads then meet in

@@ -271,16 +271,16 @@ int slots_rows(int slots_per_lane) {
     switch (slots_per_lane) {
         case 16: return slots_of<T, G, 16, ATTEND, 16>();
         case 8: return slots_of<T, G, 8, ATTEND, 16>();
+        case 6: return slots_of<T, G, 6, ATTEND, 16>();
         default: break;
     }
     if constexpr (ATTEND) {
         switch (slots_per_lane) {
+            case 4: return slots_of<T, G, 4, true, 16>();
+            case 5: return slots_of<T, G, 5, true, 16>();
             case 1: return slots_of<T, G, 1, true, 16>();
             case 2: return slots_of<T, G, 2, true, 16>();
             case 3: return slots_of<T, G, 3, true, 16>();
-            case 4: return slots_of<T, G, 4, true, 16>();
-            case 5: return slots_of<T, G, 5, true, 16>();
-            case 6: return slots_of<T, G, 6, true, 16>();
             case 7: return slots_of<T, G, 7, true, 16>();
             case 9: return slots_of<T, G, 9, true, 16>();
             case 10: return slots_of<T, G, 10, true, 16>();
@@ -301,7 +301,7 @@ int slots_rows(int slots_per_lane) {
 // 40k rows, 16 of 2560: 14.7 against 16.0 with 10 of 4096; more than 16 blocks measured slower again,
 // and so did more than 8 rows per lane, which therefore only come in where fewer, larger blocks are
 // what it takes to keep the grid resident: batch 8 at 32k rows).  Without the attention (LRU table):
-// 4096 rows where that fits, else 8192.
+// 4096 rows where that fits (3072 in the case described below), else 8192.
 template <typename T, int G, bool ATTEND>
 int pick_rows(int64_t n, int64_t heads) {
     if (n < 1) n = 1;
@@ -318,7 +318,17 @@ int pick_rows(int64_t n, int64_t heads) {
     else if (ATTEND) {
         for (int f : FS_FLAVOURS)
             if (spl == 0 && fits(f)) spl = f;
-    } else spl = fits(8) ? 8 : fits(16) ? 16 : 0;
+    } else {
+        // many workgroups per compute unit here (large batches): blocks of 3072 rows where they need
+        // no more rounds of workgroups over the device than blocks of 4096 (C3: 768 workgroups, three
+        // per compute unit, 15.6 us against 17.3 with 640 of 4096 rows)
+        spl = fits(8) ? 8 : fits(16) ? 16 : 0;
+        if (spl == 8 && fits(6)) {
+            const int64_t cus = sl_compute_units();
+            const int64_t w6 = heads * ((n + 3071) / 3072), w8 = heads * ((n + 4095) / 4096);
+            if (cus > 0 && (w6 + cus - 1) / cus <= (w8 + cus - 1) / cus) spl = 6;
+        }
+    }
     return spl == 0 && unknown ? -1 : 512 * spl;
 }
 
@@ -329,6 +339,7 @@ int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, 
     switch (rows / 512) {
         case 16: return launch_rows<T, G, 16, ATTEND, 16>(fa, sa, aa, s);
         case 8: return launch_rows<T, G, 8, ATTEND, 16>(fa, sa, aa, s);
+        case 6: return launch_rows<T, G, 6, ATTEND, 16>(fa, sa, aa, s);
         default: break;
     }
     if constexpr (ATTEND) {
@@ -338,7 +349,6 @@ int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, 
             case 3: return launch_rows<T, G, 3, true, 16>(fa, sa, aa, s);
             case 4: return launch_rows<T, G, 4, true, 16>(fa, sa, aa, s);
             case 5: return launch_rows<T, G, 5, true, 16>(fa, sa, aa, s);
-            case 6: return launch_rows<T, G, 6, true, 16>(fa, sa, aa, s);
             case 7: return launch_rows<T, G, 7, true, 16>(fa, sa, aa, s);
             case 9: return launch_rows<T, G, 9, true, 16>(fa, sa, aa, s);
             case 10: return launch_rows<T, G, 10, true, 16>(fa, sa, aa, s);
