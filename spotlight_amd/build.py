@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libspotlight_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 
-SOURCES = ["pack.hip", "hamming.hip", "topk.hip", "attn.hip", "select_attend.hip", "fused_step.hip", "fused_step_f32.hip", "fused_step_bf16.hip", "fused_step_f16.hip", "hash.hip", "hash_rows.hip", "cache.hip", "decode.hip"]
+SOURCES = ["pack.hip", "hamming.hip", "topk.hip", "attn.hip", "select_attend.hip", "fused_step.hip", "fused_step_f32_g1.hip", "fused_step_f32_g2.hip", "fused_step_f32_g4.hip", "fused_step_f32_g5.hip", "fused_step_bf16_g1.hip", "fused_step_bf16_g2.hip", "fused_step_bf16_g4.hip", "fused_step_bf16_g5.hip", "fused_step_f16_g1.hip", "fused_step_f16_g2.hip", "fused_step_f16_g4.hip", "fused_step_f16_g5.hip", "hash.hip", "hash_rows.hip", "cache.hip", "decode.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",

@@ -17,7 +17,8 @@ struct attn_args {
     uint32_t *counter;      // workspace: [B*KH] arrival tickets, left at zero
     int32_t *bump_lens;     // optional [B]: incremented once per call
     uint32_t *bump_step;    // optional [1]: incremented once per call
-    uint32_t *peer_flag;    // optional [B*KH][16]: flags of the runs of a (b, kv head), cleared by the workgroup that merges them
+    uint32_t *peer_flag;    // optional [B*KH][peer_flag_stride]: flags of the runs of a (b, kv head), cleared by the workgroup that merges them
+    int peer_flag_stride;
     int dtype, B, QH, KH, k;
     int rows;               // ranks per workgroup, a multiple of 64 (0 = choose)
     int64_t q_stride_b, kv_stride_b, kv_stride_n, kv_stride_h;

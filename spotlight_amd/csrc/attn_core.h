@@ -503,7 +503,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         }
     }
-    if (a.peer_flag && tid < S) st_agent(&a.peer_flag[static_cast<int64_t>(bh) * AT_MAX_SPLITS + tid], 0u);
+    if (a.peer_flag && tid < S) st_agent(&a.peer_flag[static_cast<int64_t>(bh) * a.peer_flag_stride + tid], 0u);
     if (tid == 0) {
         st_agent(&a.counter[bh], 0u);
         if (a.bump_lens && h == 0) a.bump_lens[b] += 1;

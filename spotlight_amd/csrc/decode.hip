@@ -58,7 +58,7 @@ ws_layout layout(const sl_decode_params &p) {
     L.n_rows = off; off += sl_align_up(sizeof(int32_t) * p.B, 256);
     // head-major codes: the flags and published histograms of the one-launch scorer + tail (the flags
     // must stay zero between calls, like the tickets); no score array, no global histogram copies
-    L.fused = off;  off += p.codes_head_major ? sl_fused_ws_bytes(p.B, p.KH) : 0;
+    L.fused = off;  off += p.codes_head_major ? sl_fused_ws_bytes(p.B, p.KH, sl_fused_peer_cap(p.n_cap)) : 0;
     L.select = off; off += p.codes_head_major ? 0 : sl_select_ws_bytes(p.B, p.KH, static_cast<int>(G * p.nbits + 1), p.n_cap);
     L.score = off;  off += p.codes_head_major ? 0 : sl_align_up(sizeof(int16_t) * p.B * p.KH * static_cast<size_t>(p.n_cap), 256);
     L.lru_fetch = off; off += p.lru_C > 0 ? sl_align_up(sizeof(int32_t) * p.B * p.KH * static_cast<size_t>(p.k), 256) : 0;
@@ -144,14 +144,14 @@ extern "C" size_t sl_decode_workspace_bytes(const sl_decode_params *p) {
 
 extern "C" size_t sl_decode_error_offset(const sl_decode_params *p) {
     if (!p || !p->codes_head_major || p->B <= 0 || p->KH <= 0) return static_cast<size_t>(-1);
-    return layout(*p).fused + sizeof(uint32_t) * static_cast<size_t>(p->B) * p->KH * FS_MAX_PEERS;
+    return layout(*p).fused + sizeof(uint32_t) * static_cast<size_t>(p->B) * p->KH * sl_fused_peer_cap(p->n_cap);
 }
 
 extern "C" int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int k, int with_lru) {
     SL_REQUIRE(B > 0 && QH > 0 && KH > 0 && QH % KH == 0 && nbits > 0 && nbits % 32 == 0 && n_max > 0 && k > 0, SL_ERR_SHAPE);
     const int G = QH / KH;
     if (!sl_fused_step_supported(G, nbits / 32, G * nbits + 1, n_max, B, KH)) return 0;
-    const int rows = sl_fused_step_rows(dtype, G, !with_lru, n_max, B, KH);
+    const int rows = sl_fused_step_rows(dtype, G, !with_lru, n_max, B, KH, sl_fused_peer_cap(n_max));
     return rows > 0 ? rows : 0;
 }
 
@@ -233,6 +233,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
             fused_args fa{};
             fa.q_code = q_code; fa.k_code = p.codes; fa.q_stride_b = static_cast<int64_t>(p.QH) * W;
             fa.k_stride_b = p.n_cap * p.KH * W; fa.k_stride_h = p.n_cap * W; fa.head_map = p.head_map;
+            fa.peer_cap = sl_fused_peer_cap(p.n_cap);
             select_args fs{};
             fs.B = p.B; fs.KH = p.KH; fs.n_bins = G * p.nbits + 1; fs.idx = p.idx; fs.seq_lens = n_rows;
             fs.k = p.k; fs.len_bias = 0; fs.n = p.n_max;

@@ -29,10 +29,10 @@ int g_fused_rows = 0;  // sl_tune("fused_rows", 0 | multiple of 512): rows per b
 static uint32_t g_fused_spin_limit = FS_SPIN_LIMIT;
 static int g_fused_phantom_peer = 0;
 
-size_t sl_fused_ws_bytes(int B, int KH) {
+size_t sl_fused_ws_bytes(int B, int KH, int peer_cap) {
     const size_t bh = static_cast<size_t>(B) * KH;
-    return sl_align_up(sizeof(uint32_t) * (bh * FS_MAX_PEERS + 64), 256) +           // flags, then the error word
-           sl_align_up(sizeof(uint32_t) * bh * FS_MAX_PEERS * FS_NB_PAD, 256);       // published histograms
+    return sl_align_up(sizeof(uint32_t) * (bh * peer_cap + 64), 256) +           // flags, then the error word
+           sl_align_up(sizeof(uint32_t) * bh * peer_cap * FS_NB_PAD, 256);       // published histograms
 }
 
 int sl_fused_tune(const char *key, int value) {
@@ -42,18 +42,40 @@ int sl_fused_tune(const char *key, int value) {
     return SL_ERR_UNSUPPORTED;
 }
 
-int sl_fused_step_rows(int dtype, int G, bool attend, int64_t n, int B, int KH) {
-    const int64_t heads = static_cast<int64_t>(B) * KH;
-    switch (dtype) {
-        case SL_F32: return sl_fused_pick_f32(G, attend, n, heads);
-        case SL_BF16: return sl_fused_pick_bf16(G, attend, n, heads);
-        case SL_F16: return sl_fused_pick_f16(G, attend, n, heads);
-        default: return 0;
+namespace {
+
+#define SL_FUSED_BY_G(name, what, ...)              \
+    switch (G) {                                    \
+        case 1: return what##_##name##_g1(__VA_ARGS__); \
+        case 2: return what##_##name##_g2(__VA_ARGS__); \
+        case 4: return what##_##name##_g4(__VA_ARGS__); \
+        case 5: return what##_##name##_g5(__VA_ARGS__); \
+        default: return SL_ERR_UNSUPPORTED;         \
     }
+
+int pick_f32(int G, bool attend, int64_t n, int64_t heads, int cap) { SL_FUSED_BY_G(f32, sl_fused_pick, attend, n, heads, cap) }
+int pick_bf16(int G, bool attend, int64_t n, int64_t heads, int cap) { SL_FUSED_BY_G(bf16, sl_fused_pick, attend, n, heads, cap) }
+int pick_f16(int G, bool attend, int64_t n, int64_t heads, int cap) { SL_FUSED_BY_G(f16, sl_fused_pick, attend, n, heads, cap) }
+int launch_f32(int G, const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s) { SL_FUSED_BY_G(f32, sl_fused_launch, fa, sa, aa, attend, s) }
+int launch_bf16(int G, const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s) { SL_FUSED_BY_G(bf16, sl_fused_launch, fa, sa, aa, attend, s) }
+int launch_f16(int G, const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s) { SL_FUSED_BY_G(f16, sl_fused_launch, fa, sa, aa, attend, s) }
+
+}  // namespace
+
+int sl_fused_step_rows(int dtype, int G, bool attend, int64_t n, int B, int KH, int peer_cap) {
+    const int64_t heads = static_cast<int64_t>(B) * KH;
+    int rows = 0;
+    switch (dtype) {
+        case SL_F32: rows = pick_f32(G, attend, n, heads, peer_cap); break;
+        case SL_BF16: rows = pick_bf16(G, attend, n, heads, peer_cap); break;
+        case SL_F16: rows = pick_f16(G, attend, n, heads, peer_cap); break;
+        default: break;
+    }
+    return rows == SL_ERR_UNSUPPORTED ? 0 : rows;
 }
 
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH) {
-    return (G == 1 || G == 2 || G == 4) && W == 4 && n_bins <= 1024 && n_bins <= FS_NB_PAD &&
+    return (G == 1 || G == 2 || G == 4 || G == 5) && W == 4 && n_bins <= 1024 && n_bins <= FS_NB_PAD &&
            (n + 8191) / 8192 <= FS_MAX_PEERS && B <= 65535 && KH <= 65535;
 }
 
@@ -66,17 +88,19 @@ int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool atten
                (fa.q_stride_b % 4) == 0, SL_ERR_ALIGN);
     int rc = sl_attn_prepare(aa, attn_ws, attn_ws_bytes);
     if (rc != SL_OK) return rc;
+    SL_REQUIRE(fa.peer_cap == 16 || fa.peer_cap == 32, SL_ERR_SHAPE);
     const size_t bh = static_cast<size_t>(aa.B) * aa.KH;
     fa.peer_flag = static_cast<uint32_t *>(fused_ws);
-    fa.error = fa.peer_flag + bh * FS_MAX_PEERS;
-    fa.peer_hist = reinterpret_cast<uint32_t *>(static_cast<char *>(fused_ws) + sl_align_up(sizeof(uint32_t) * (bh * FS_MAX_PEERS + 64), 256));
+    fa.error = fa.peer_flag + bh * fa.peer_cap;
+    fa.peer_hist = reinterpret_cast<uint32_t *>(static_cast<char *>(fused_ws) + sl_align_up(sizeof(uint32_t) * (bh * fa.peer_cap + 64), 256));
     aa.peer_flag = fa.peer_flag;
+    aa.peer_flag_stride = fa.peer_cap;
     fa.spin_limit = g_fused_spin_limit;
     fa.phantom_peers = g_fused_phantom_peer;   // (the launcher drops it where a head has no free flag)
     switch (aa.dtype) {
-        case SL_F32: return sl_fused_launch_f32(fa, sa, aa, attend, s);
-        case SL_BF16: return sl_fused_launch_bf16(fa, sa, aa, attend, s);
-        case SL_F16: return sl_fused_launch_f16(fa, sa, aa, attend, s);
+        case SL_F32: return launch_f32(G, fa, sa, aa, attend, s);
+        case SL_BF16: return launch_bf16(G, fa, sa, aa, attend, s);
+        case SL_F16: return launch_f16(G, fa, sa, aa, attend, s);
         default: return SL_ERR_UNSUPPORTED;
     }
 }

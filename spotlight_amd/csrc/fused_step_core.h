@@ -15,7 +15,7 @@ constexpr int FS_NW = 8;
 constexpr int FS_THREADS = FS_NW * 64;
 constexpr int FS_MAX_BPT = 2;                        // histogram bins per lane (<= 1024 bins: sl_fused_step_supported)
 
-static_assert(FS_MAX_PEERS == AT_MAX_SPLITS, "one attention run per block of rows");
+static_assert(FS_MAX_PEERS == AT_PART_SPLITS, "one attention run per block of rows");
 
 // FS_SLOTS rows per lane (row = block start + wave * 64 FS_SLOTS + slot * 64 + lane): blocks of
 // 512 FS_SLOTS rows; pick_rows chooses the size by shape.
@@ -25,7 +25,7 @@ static_assert(FS_MAX_PEERS == AT_MAX_SPLITS, "one attention run per block of row
 template <typename T, int G, int FS_SLOTS, bool ATTEND, int MAXS>
 __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_args fa, select_args sa, attn_args aa) {
     constexpr int W = 4;
-    static_assert(MAXS == 16, "peers polled by the lanes of one wave; merge flavour");
+    static_assert(MAXS == 16 || MAXS == 32, "peers polled by the lanes of one wave; merge flavours");
     constexpr int FS_BLOCK = FS_THREADS * FS_SLOTS;
     __shared__ uint32_t s_wave[64];
     __shared__ int s_tn[4];
@@ -109,8 +109,8 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     int lo = s_range[0], hi = s_range[1];   // a block that got here holds at least one row: lo <= hi
     uint32_t cnt[FS_MAX_BPT], before[FS_MAX_BPT], mine = 0;
     if (S > 1) {
-        uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * FS_MAX_PEERS * FS_NB_PAD;
-        uint32_t *flags = fa.peer_flag + static_cast<int64_t>(bh) * FS_MAX_PEERS;
+        uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * fa.peer_cap * FS_NB_PAD;
+        uint32_t *flags = fa.peer_flag + static_cast<int64_t>(bh) * fa.peer_cap;
         // every bin is published, zeros included: the peers read the union of all ranges
         for (int e = tid; e < NB; e += FS_THREADS) st_agent(peers + blk * FS_NB_PAD + e, s_hist[e]);
         publish_wait();
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     const int n_ranks = hi - lo + 1;
     const int BPT = (n_ranks + FS_THREADS - 1) / FS_THREADS;
     if (S > 1) {
-        const uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * FS_MAX_PEERS * FS_NB_PAD;
+        const uint32_t *peers = fa.peer_hist + static_cast<int64_t>(bh) * fa.peer_cap * FS_NB_PAD;
 #pragma unroll
         for (int j = 0; j < FS_MAX_BPT; ++j) {
             const int r = tid * BPT + j;
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
             uint32_t last = 0;
             if (lane == 0) last = arrive_last(&aa.counter[bh], static_cast<uint32_t>(S)) ? 1u : 0u;
             if (__builtin_amdgcn_readfirstlane(last)) {
-                if (lane < S) st_agent(fa.peer_flag + static_cast<int64_t>(bh) * FS_MAX_PEERS + lane, 0u);
+                if (lane < S) st_agent(fa.peer_flag + static_cast<int64_t>(bh) * fa.peer_cap + lane, 0u);
                 if (lane == 0) st_agent(&aa.counter[bh], 0u);
             }
         }
@@ -257,59 +257,83 @@ int launch_rows(fused_args fa, const select_args &sa, const attn_args &aa, hipSt
     const unsigned heads = static_cast<unsigned>(aa.B) * aa.KH;
     const int64_t n = sa.n > 0 ? sa.n : 1;
     fa.blocks = static_cast<unsigned>((n + FS_THREADS * SLOTS - 1) / (FS_THREADS * SLOTS));
-    if (fa.blocks >= FS_MAX_PEERS) fa.phantom_peers = 0;   // a phantom peer needs a free flag
+    if (fa.blocks >= static_cast<unsigned>(MAXS < fa.peer_cap ? MAXS : fa.peer_cap)) fa.phantom_peers = 0;   // a phantom peer needs a free flag
     const dim3 grid(ATTEND ? xcd_grid(heads, fa.blocks) : heads * fa.blocks);
     score_select_attend_kernel<T, G, SLOTS, ATTEND, MAXS><<<grid, dim3(FS_THREADS), 0, s>>>(fa, sa, aa);
     return sl_check_launch();
 }
 
-// Rows per block come in multiples of 512 (one row per lane): the flavours that exist.
+// Rows per block come in multiples of 512 (one row per lane): the flavours that exist.  Those of 8 and
+// more rows per lane also exist for up to 32 blocks per head (caches beyond 64k rows).
 constexpr int FS_FLAVOURS[] = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 14, 16};
 
+#define FS_FOR_FLAVOUR(spl, many, CALL)                                 \
+    if (many) {                                                         \
+        if constexpr (ATTEND) {                                         \
+            switch (spl) {                                              \
+                case 8: return CALL(8, true, 32);                       \
+                case 9: return CALL(9, true, 32);                       \
+                case 10: return CALL(10, true, 32);                     \
+                case 11: return CALL(11, true, 32);                     \
+                case 12: return CALL(12, true, 32);                     \
+                case 14: return CALL(14, true, 32);                     \
+                case 16: return CALL(16, true, 32);                     \
+                default: break;                                         \
+            }                                                           \
+        }                                                               \
+    } else {                                                            \
+        switch (spl) {                                                  \
+            case 16: return CALL(16, ATTEND, 16);                       \
+            case 8: return CALL(8, ATTEND, 16);                         \
+            case 6: return CALL(6, ATTEND, 16);                         \
+            default: break;                                             \
+        }                                                               \
+        if constexpr (ATTEND) {                                         \
+            switch (spl) {                                              \
+                case 1: return CALL(1, true, 16);                       \
+                case 2: return CALL(2, true, 16);                       \
+                case 3: return CALL(3, true, 16);                       \
+                case 4: return CALL(4, true, 16);                       \
+                case 5: return CALL(5, true, 16);                       \
+                case 7: return CALL(7, true, 16);                       \
+                case 9: return CALL(9, true, 16);                       \
+                case 10: return CALL(10, true, 16);                     \
+                case 11: return CALL(11, true, 16);                     \
+                case 12: return CALL(12, true, 16);                     \
+                case 14: return CALL(14, true, 16);                     \
+                default: break;                                         \
+            }                                                           \
+        }                                                               \
+    }
+
 template <typename T, int G, bool ATTEND>
-int slots_rows(int slots_per_lane) {
-    switch (slots_per_lane) {
-        case 16: return slots_of<T, G, 16, ATTEND, 16>();
-        case 8: return slots_of<T, G, 8, ATTEND, 16>();
-        case 6: return slots_of<T, G, 6, ATTEND, 16>();
-        default: break;
-    }
-    if constexpr (ATTEND) {
-        switch (slots_per_lane) {
-            case 4: return slots_of<T, G, 4, true, 16>();
-            case 5: return slots_of<T, G, 5, true, 16>();
-            case 1: return slots_of<T, G, 1, true, 16>();
-            case 2: return slots_of<T, G, 2, true, 16>();
-            case 3: return slots_of<T, G, 3, true, 16>();
-            case 7: return slots_of<T, G, 7, true, 16>();
-            case 9: return slots_of<T, G, 9, true, 16>();
-            case 10: return slots_of<T, G, 10, true, 16>();
-            case 11: return slots_of<T, G, 11, true, 16>();
-            case 12: return slots_of<T, G, 12, true, 16>();
-            case 14: return slots_of<T, G, 14, true, 16>();
-            default: break;
-        }
-    }
+int slots_rows(int slots_per_lane, bool many) {
+#define FS_SLOTS_CALL(SPL, ATT, MX) slots_of<T, G, SPL, ATT, MX>()
+    FS_FOR_FLAVOUR(slots_per_lane, many, FS_SLOTS_CALL)
+#undef FS_SLOTS_CALL
     return -1;
 }
 
 // Rows per block for a launch over n rows, 0 = the shape cannot take this launch on this device, -1 = the
-// runtime could not tell.  Every workgroup must be resident at once (they wait for their peers) and a
-// (b, kv head) has at most 16 blocks.  With the attention in the launch: the smallest blocks that
-// satisfy both -- more, lighter workgroups per head (measured at batch 1: 8k rows, 9 blocks of 1024:
-// 11.3 us against 14.1 with 2 of 4096; 32k rows, 13 blocks of 2560: 14.1 against 15.5 with 9 of 4096;
-// 40k rows, 16 of 2560: 14.7 against 16.0 with 10 of 4096; more than 16 blocks measured slower again,
-// and so did more than 8 rows per lane, which therefore only come in where fewer, larger blocks are
-// what it takes to keep the grid resident: batch 8 at 32k rows).  Without the attention (LRU table):
-// 4096 rows where that fits (3072 in the case described below), else 8192.
+// runtime could not tell.  Every workgroup must be resident at once (they wait for their peers).  A
+// (b, kv head) has at most 16 blocks up to 64k rows, at most peer_cap (32 in a workspace laid out for a
+// longer cache) beyond.  With the attention in the launch: the smallest blocks that satisfy both --
+// more, lighter workgroups per head (measured at batch 1: 8k rows, 9 blocks of 1024: 11.3 us against
+// 14.1 with 2 of 4096; 32k rows, 13 blocks of 2560: 14.1 against 15.5 with 9 of 4096; 40k rows, 16 of
+// 2560: 14.7 against 16.0 with 10 of 4096; up to 64k rows more than 16 blocks measured slower again, and
+// so did more than 8 rows per lane, which therefore only come in where fewer, larger blocks are what it
+// takes to keep the grid resident: batch 8 at 32k rows; 128k rows: 29 blocks of 4608 rows 24.6 us
+// against 30.2 with 17 of 8192).  Without the attention (LRU table): 4096 rows where that fits (3072 in
+// the case described below), else 8192.
 template <typename T, int G, bool ATTEND>
-int pick_rows(int64_t n, int64_t heads) {
+int pick_rows(int64_t n, int64_t heads, int peer_cap) {
     if (n < 1) n = 1;
     bool unknown = false;
+    const int64_t most = n <= 16 * 4096 || peer_cap < 32 ? 16 : 32;
     auto fits = [&](int spl) {
         const int64_t rows = 512 * spl, blocks = (n + rows - 1) / rows;
-        if (blocks > FS_MAX_PEERS) return false;
-        const int slots = slots_rows<T, G, ATTEND>(spl);
+        if (blocks > most) return false;
+        const int slots = slots_rows<T, G, ATTEND>(spl, blocks > 16);
         if (slots == 0) unknown = true;
         return heads * blocks <= slots;
     };
@@ -334,51 +358,24 @@ int pick_rows(int64_t n, int64_t heads) {
 
 template <typename T, int G, bool ATTEND>
 int launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, hipStream_t s) {
-    const int rows = pick_rows<T, G, ATTEND>(sa.n, static_cast<int64_t>(aa.B) * aa.KH);
+    const int rows = pick_rows<T, G, ATTEND>(sa.n, static_cast<int64_t>(aa.B) * aa.KH, fa.peer_cap);
     if (rows < 0) return SL_ERR_LAUNCH;
-    switch (rows / 512) {
-        case 16: return launch_rows<T, G, 16, ATTEND, 16>(fa, sa, aa, s);
-        case 8: return launch_rows<T, G, 8, ATTEND, 16>(fa, sa, aa, s);
-        case 6: return launch_rows<T, G, 6, ATTEND, 16>(fa, sa, aa, s);
-        default: break;
-    }
-    if constexpr (ATTEND) {
-        switch (rows / 512) {
-            case 1: return launch_rows<T, G, 1, true, 16>(fa, sa, aa, s);
-            case 2: return launch_rows<T, G, 2, true, 16>(fa, sa, aa, s);
-            case 3: return launch_rows<T, G, 3, true, 16>(fa, sa, aa, s);
-            case 4: return launch_rows<T, G, 4, true, 16>(fa, sa, aa, s);
-            case 5: return launch_rows<T, G, 5, true, 16>(fa, sa, aa, s);
-            case 7: return launch_rows<T, G, 7, true, 16>(fa, sa, aa, s);
-            case 9: return launch_rows<T, G, 9, true, 16>(fa, sa, aa, s);
-            case 10: return launch_rows<T, G, 10, true, 16>(fa, sa, aa, s);
-            case 11: return launch_rows<T, G, 11, true, 16>(fa, sa, aa, s);
-            case 12: return launch_rows<T, G, 12, true, 16>(fa, sa, aa, s);
-            case 14: return launch_rows<T, G, 14, true, 16>(fa, sa, aa, s);
-            default: break;
-        }
-    }
+    if (rows == 0) return SL_ERR_UNSUPPORTED;
+    const bool many = ((sa.n > 0 ? sa.n : 1) + rows - 1) / rows > 16;
+#define FS_LAUNCH_CALL(SPL, ATT, MX) launch_rows<T, G, SPL, ATT, MX>(fa, sa, aa, s)
+    FS_FOR_FLAVOUR(rows / 512, many, FS_LAUNCH_CALL)
+#undef FS_LAUNCH_CALL
     return SL_ERR_UNSUPPORTED;
 }
 
-template <typename T>
-int fused_launch_t(const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s) {
-    switch (aa.QH / aa.KH) {
-        case 1: return attend ? launch_tg<T, 1, true>(fa, sa, aa, s) : launch_tg<T, 1, false>(fa, sa, aa, s);
-        case 2: return attend ? launch_tg<T, 2, true>(fa, sa, aa, s) : launch_tg<T, 2, false>(fa, sa, aa, s);
-        case 4: return attend ? launch_tg<T, 4, true>(fa, sa, aa, s) : launch_tg<T, 4, false>(fa, sa, aa, s);
-        default: return SL_ERR_UNSUPPORTED;
-    }
+template <typename T, int G>
+int fused_launch_tg(const fused_args &fa, const select_args &sa, const attn_args &aa, bool attend, hipStream_t s) {
+    return attend ? launch_tg<T, G, true>(fa, sa, aa, s) : launch_tg<T, G, false>(fa, sa, aa, s);
 }
 
-template <typename T>
-int fused_pick_t(int G, bool attend, int64_t n, int64_t heads) {
-    switch (G) {
-        case 1: return attend ? pick_rows<T, 1, true>(n, heads) : pick_rows<T, 1, false>(n, heads);
-        case 2: return attend ? pick_rows<T, 2, true>(n, heads) : pick_rows<T, 2, false>(n, heads);
-        case 4: return attend ? pick_rows<T, 4, true>(n, heads) : pick_rows<T, 4, false>(n, heads);
-        default: return 0;
-    }
+template <typename T, int G>
+int fused_pick_tg(bool attend, int64_t n, int64_t heads, int peer_cap) {
+    return attend ? pick_rows<T, G, true>(n, heads, peer_cap) : pick_rows<T, G, false>(n, heads, peer_cap);
 }
 
 }  // namespace

@@ -98,10 +98,10 @@ class LayerDecodeState:
         # takes head-major whenever that launch covers the shape.  ``codes`` is always indexed
         # [b, row, kv head, word]; with head-major storage it is a strided view.
         if codes_layout == "auto":
-            # without an LRU table the launch also attends, one run per block of rows (9 to 24 blocks of
-            # 1024 ... 8192 rows): keep <= 128 rows per block on average (and stay with the three launches
-            # beyond 64k rows: measured no faster there)
-            rows_ok = bool(lru_slots) or (k <= 128 * min(16, (n_cap + 1023) // 1024) and n_cap <= 65536)
+            # without an LRU table the launch also attends, one run per block of rows (up to 16 blocks per head,
+            # 32 beyond 64k rows): keep <= 128 rows per block on average
+            most_blocks = min(32 if n_cap > 65536 else 16, (n_cap + 511) // 512)
+            rows_ok = bool(lru_slots) or k <= 128 * most_blocks
             fits = 0
             if rows_ok and W == 4:
                 # all blocks of a launch must be resident at once; the library knows what the device holds

@@ -324,7 +324,7 @@ def test_decode_many_blocks_and_long_cache(env):
                           (40000, 200, "head"), (60000, 300, "head"), (70000, 300, "auto"), (140000, 500, "auto"), (270000, 64, "auto")):
         g = _gen(n0)
         st = _make_state(decode, g, 1, 8, 2, n0, (n0 + 64 + 7) // 8 * 8, k, torch.bfloat16, codes_layout=layout)
-        assert st.codes_layout == ("token" if n0 > 65000 else layout if layout != "auto" else "head")
+        assert st.codes_layout == ("token" if n0 > 262144 else layout if layout != "auto" else "head")
         for step in range(2):
             q = torch.randn(1, 8, 128, generator=g).to(torch.bfloat16)
             kn = torch.randn(1, 2, 128, generator=g).to(torch.bfloat16)
