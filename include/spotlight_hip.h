@@ -284,7 +284,8 @@ typedef struct {
     const void *w1_k, *b1_k, *w2_k, *b2_k;   /* [KH, ...]                       */
     /* caches, token-major; codes_head_major != 0: codes are [B, KH, n_cap, W]  */
     /* and scorer, selection and (without an LRU table) attention run as ONE    */
-    /* launch; needs W == 4, QH/KH in {1,2,4}, n_max <= 131072 and a grid that  */
+    /* launch; needs W == 4, QH/KH in {1,2,4,5}, n_max <= 262144 (131072 with   */
+    /* an LRU table) and a grid that                                            */
     /* fits the device at once (sl_decode_head_major_fits): otherwise           */
     /* SL_ERR_UNSUPPORTED, use token-major codes.  The blocks of that launch    */
     /* wait for each other (bounded; see sl_decode_error_offset), which assumes */
