@@ -312,6 +312,16 @@ typedef struct {
     /* scratch */
     void *ws;
     size_t ws_bytes;
+    /* Budget rule evaluated on the device (budget_on != 0): a sequence that holds  */
+    /* n rows after this step's append keeps                                        */
+    /*   max(min(n, budget_min_remain), n - int(n * budget_mask_out))               */
+    /* rows (spotlight_generation.py:162-164; the product in double precision,      */
+    /* truncated like Python's int()), capped at k.  k is then only the row length  */
+    /* of idx and the cap: entries of an idx row beyond the budget are -1, and one  */
+    /* captured graph stays valid while the budget grows with the cache.            */
+    int budget_on;
+    int budget_min_remain;
+    double budget_mask_out;
 } sl_decode_params;
 
 size_t sl_decode_workspace_bytes(const sl_decode_params *p);

@@ -38,6 +38,7 @@ class DecodeParams(C.Structure):
         ("k_res", c_void_p), ("v_res", c_void_p), ("slots_out", c_void_p),
         ("lru_stats", c_void_p), ("step_counter", c_void_p),
         ("ws", c_void_p), ("ws_bytes", c_size_t),
+        ("budget_on", c_int), ("budget_min_remain", c_int), ("budget_mask_out", C.c_double),
     ]
 
 

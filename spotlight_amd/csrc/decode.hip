@@ -55,7 +55,7 @@ ws_layout layout(const sl_decode_params &p) {
     size_t off = 0;
     L.q_code = off; off += sl_align_up(sizeof(uint32_t) * p.B * p.QH * W, 256);
     L.attn = off;   off += sl_align_up(sl_attn_ws_bytes(p.B, p.QH, p.KH, 1), 256);  // does not depend on k
-    L.n_rows = off; off += sl_align_up(sizeof(int32_t) * p.B, 256);
+    L.n_rows = off; off += sl_align_up(sizeof(int32_t) * 2 * p.B, 256);   // row counts, then rows to keep, per sequence
     // head-major codes: the flags and published histograms of the one-launch scorer + tail (the flags
     // must stay zero between calls, like the tickets); no score array, no global histogram copies
     L.fused = off;  off += p.codes_head_major ? sl_fused_ws_bytes(p.B, p.KH, sl_fused_peer_cap(p.n_cap)) : 0;
@@ -76,6 +76,7 @@ int validate(const sl_decode_params &p) {
     SL_REQUIRE(p.q && p.k_new && p.v_new && p.codes && p.keys && p.vals && p.seq_lens && p.out && p.idx, SL_ERR_NULL);
     SL_REQUIRE(p.w1_q && p.w1_k, SL_ERR_NULL);
     if (p.rope_inv_freq) SL_REQUIRE(p.q_rot && sl_aligned(p.q_rot, 16), SL_ERR_NULL);
+    if (p.budget_on) SL_REQUIRE(p.budget_mask_out >= 0.0 && p.budget_mask_out <= 1.0 && p.budget_min_remain >= 0, SL_ERR_SHAPE);
     if (p.lru_C > 0)
         SL_REQUIRE(p.slot_token && p.slot_stamp && p.token_slot && p.k_res && p.v_res && p.slots_out && p.step_counter, SL_ERR_NULL);
     return SL_OK;
@@ -178,6 +179,10 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     // seq_lens at its end.  No launch reads a word that one of its own workgroups writes.  (A subset
     // of stages without the hash launch works on the row counts the last hash launch left.)
     int32_t *n_rows = reinterpret_cast<int32_t *>(ws + L.n_rows);
+    // With a budget rule the hash launch also leaves, per sequence, the rows this step keeps (k stays the
+    // row length of idx and the cap); the selection reads it, everything after the selection skips the -1
+    // entries that fill the rest of an idx row.
+    int32_t *keep_rows = p.budget_on ? n_rows + p.B : nullptr;
     const size_t attn_bytes = L.n_rows - L.attn;
 
     // 1. hash q and the new key; append code, K, V
@@ -225,6 +230,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         const int one = SL_STAGE_SCORE | SL_STAGE_SELECT | (attend ? SL_STAGE_ATTN : 0);
         SL_REQUIRE((stages & one) == 0 || (stages & one) == one, SL_ERR_UNSUPPORTED);
         ha.len_out = n_rows;
+        ha.keep_out = keep_rows; ha.keep_mask_out = p.budget_mask_out; ha.keep_min = p.budget_min_remain;
         if (stages & SL_STAGE_HASH) {
             rc = sl_hash_launch(ha, s);
             if (rc != SL_OK) return rc;
@@ -235,7 +241,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
             fa.k_stride_b = p.n_cap * p.KH * W; fa.k_stride_h = p.n_cap * W; fa.head_map = p.head_map;
             fa.peer_cap = sl_fused_peer_cap(p.n_cap);
             select_args fs{};
-            fs.B = p.B; fs.KH = p.KH; fs.n_bins = G * p.nbits + 1; fs.idx = p.idx; fs.seq_lens = n_rows;
+            fs.B = p.B; fs.KH = p.KH; fs.n_bins = G * p.nbits + 1; fs.idx = p.idx; fs.seq_lens = n_rows; fs.keep = keep_rows;
             fs.k = p.k; fs.len_bias = 0; fs.n = p.n_max;
             rc = sl_fused_step_launch(fa, fs, aa, attend, ws + L.fused, ws + L.attn, attn_bytes, s);
             if (rc != SL_OK || attend) return rc;
@@ -253,6 +259,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         ha.zero_count = static_cast<int64_t>(ta.n_bins) * ta.hist_used;
         ha.zero_stride = static_cast<int64_t>(ta.n_bins) * ta.hist_groups;
         ha.len_out = n_rows;
+        ha.keep_out = keep_rows; ha.keep_mask_out = p.budget_mask_out; ha.keep_min = p.budget_min_remain;
         // 2. score seq_lens[b] + 1 rows
         hamming_args sa{};
         sa.q_code = q_code; sa.k_code = p.codes; sa.out = score; sa.hist = ta.hist; sa.hist_groups = ta.hist_groups; sa.hist_span = ta.hist_span; sa.seq_lens = n_rows;
@@ -269,7 +276,7 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         }
 
         // 3. select
-        ta.score = score; ta.idx = p.idx; ta.seq_lens = n_rows;
+        ta.score = score; ta.idx = p.idx; ta.seq_lens = n_rows; ta.keep = keep_rows;
         ta.k = p.k; ta.len_bias = 0; ta.n = p.n_max;
         ta.stride_b = p.KH * p.n_cap; ta.stride_n = 1; ta.stride_h = p.n_cap;
         // 3. select -- or 3+5 in one launch when there is no LRU in between and the shapes allow

@@ -24,8 +24,9 @@ struct fused_args {
 
 size_t sl_fused_ws_bytes(int B, int KH, int peer_cap);
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH);
-// rows per block the launch would use on the current device for this shape (its workgroups wait for each
-// other, so all of them must be resident at once); 0: the shape cannot take this launch, -1: unknown
+// rows per block the launch would use on the current device for this shape (the blocks of a head wait for
+// each other, so a head's blocks must fit one XCD's share of the device); 0: the shape cannot take this
+// launch, -1: unknown
 int sl_fused_step_rows(int dtype, int G, bool attend, int64_t n, int B, int KH, int peer_cap);
 // sa: n_bins, k, idx, seq_lens (row counts), len_bias, n, B, KH; aa as for sl_attn_launch (aa.idx is ignored).
 // attend false: the launch stops at the list of kept rows (sa.idx); of aa only the shape and the tickets are used.

@@ -2,11 +2,11 @@
 // when the key codes are stored head-major (behind an LRU table the launch ends at the selection).
 //
 // With codes laid out [B, KH, n_cap, W] a workgroup can own a block of 4096 rows of ONE (b, kv head)
-// (8192 rows, 16 per lane, when that is what it takes for all blocks to be resident):
+// (512 to 8192 rows, 1 to 16 per lane, by shape):
 // it streams the block's codes (64 KB, contiguous), keeps the 8 scores per lane in registers and
 // builds the block's score histogram in LDS.  The only thing it lacks for the selection is what the
-// other blocks of the same (b, kv head) saw, so the blocks -- at most 16, all resident at the same
-// time -- swap histograms: each publishes its 513 bins with device-coherent stores and raises a flag,
+// other blocks of the same (b, kv head) saw, so the blocks -- at most 16 (32 beyond 64k rows), running
+// at the same time -- swap histograms: each publishes its 513 bins with device-coherent stores and raises a flag,
 // waits (bounded) for the flags of its peers and reads their bins.  From there on it is the fused
 // select + attend kernel: threshold from the summed histograms, kept rows in front of the block from
 // the peers with a lower block number, placement, attention over exactly its kept rows, run merge.
@@ -14,11 +14,13 @@
 // int16 score array (written, then read back), the global histogram copies with their atomics and
 // their clearing; the swap costs about 1.2 us (measured: publish, wait for 8 peers, read 8 x 513 bins).
 //
-// Waiting on other workgroups is only safe while every workgroup of the launch can be resident at
-// once; the host checks the grid against the device's capacity for this kernel and otherwise the
-// caller must use the three-launch path (token-major codes).  The wait is bounded all the same: a
-// workgroup that gives up sets an error word and goes on, so the launch always drains (exercised
-// from the host with a short limit and a peer that does not exist, sl_tune "fused_phantom_peer").
+// Waiting on other workgroups is only safe while the workgroups waited for can start: the blocks of a
+// (b, kv head) are numbered consecutively in the order in which the device starts workgroups, and a
+// head's blocks must fit one XCD's share of the device (fused_step_core.h: pick_rows) -- the grid as a
+// whole may be larger than the device holds at once, it then runs in rounds.  The wait is bounded all
+// the same: a workgroup that gives up sets an error word and goes on, so the launch always drains
+// (exercised from the host with a short limit and a peer that does not exist, sl_tune
+// "fused_phantom_peer").
 #include "fused_step.h"
 
 #include <string.h>
@@ -36,7 +38,13 @@ size_t sl_fused_ws_bytes(int B, int KH, int peer_cap) {
 }
 
 int sl_fused_tune(const char *key, int value) {
-    if (!strcmp(key, "fused_rows") && value >= 0 && value <= 8192 && value % 512 == 0) { g_fused_rows = value; return SL_OK; }
+    if (!strcmp(key, "fused_rows")) {
+        // the block sizes that exist as kernel flavours: 512 x {1 .. 12, 14, 16}
+        const int f = value / 512;
+        if (value != 0 && (value % 512 != 0 || f < 1 || f > 16 || f == 13 || f == 15)) return SL_ERR_UNSUPPORTED;
+        g_fused_rows = value;
+        return SL_OK;
+    }
     if (!strcmp(key, "fused_spin_limit") && value >= 0) { g_fused_spin_limit = value ? static_cast<uint32_t>(value) : FS_SPIN_LIMIT; return SL_OK; }
     if (!strcmp(key, "fused_phantom_peer") && (value == 0 || value == 1)) { g_fused_phantom_peer = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;

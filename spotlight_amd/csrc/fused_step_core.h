@@ -67,11 +67,22 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
         const int64_t t = t_base + j * 64;
         kreg[j] = kb[t < sa.n ? t : sa.n - 1];
     }
-    const int64_t n_b = tokens_of(sa, b);
-    const int k_eff = n_b < sa.k ? static_cast<int>(n_b) : sa.k;
+    int64_t n_b;
+    int k_eff;
+    rows_and_keep(sa, b, n_b, k_eff);
     int32_t *out = sa.idx + static_cast<int64_t>(bh) * sa.k;
     if (blk == 0)
         for (int i = k_eff + tid; i < sa.k; i += FS_THREADS) out[i] = -1;
+    if (n_b == 0) {
+        // no rows at all (a subset of stages run before any hash launch left a row count): nothing is
+        // kept, and the attention over nothing is zero
+        if constexpr (ATTEND) {
+            T *ob = static_cast<T *>(aa.out) + (static_cast<int64_t>(b) * aa.QH + static_cast<int64_t>(h) * G) * AT_D;
+            if (blk == 0)
+                for (int e = tid; e < G * AT_D; e += FS_THREADS) ob[e] = from_f32<T>(0.f);
+        }
+        return;
+    }
     if (static_cast<int64_t>(blk) * FS_BLOCK >= n_b) return;
     const int S = static_cast<int>((n_b + FS_BLOCK - 1) / FS_BLOCK);  // blocks (= attention runs) of this (b, kv head)
 
@@ -315,30 +326,59 @@ int slots_rows(int slots_per_lane, bool many) {
 }
 
 // Rows per block for a launch over n rows, 0 = the shape cannot take this launch on this device, -1 = the
-// runtime could not tell.  Every workgroup must be resident at once (they wait for their peers).  A
-// (b, kv head) has at most 16 blocks up to 64k rows, at most peer_cap (32 in a workspace laid out for a
-// longer cache) beyond.  With the attention in the launch: the smallest blocks that satisfy both --
-// more, lighter workgroups per head (measured at batch 1: 8k rows, 9 blocks of 1024: 11.3 us against
-// 14.1 with 2 of 4096; 32k rows, 13 blocks of 2560: 14.1 against 15.5 with 9 of 4096; 40k rows, 16 of
-// 2560: 14.7 against 16.0 with 10 of 4096; up to 64k rows more than 16 blocks measured slower again, and
-// so did more than 8 rows per lane, which therefore only come in where fewer, larger blocks are what it
-// takes to keep the grid resident: batch 8 at 32k rows; 128k rows: 29 blocks of 4608 rows 24.6 us
-// against 30.2 with 17 of 8192).  Without the attention (LRU table): 4096 rows where that fits (3072 in
-// the case described below), else 8192.
+// runtime could not tell.  The blocks of a (b, kv head) wait for each other, so they must be able to run
+// at the same time.  Workgroups reach the compute units in the order of their numbers (per XCD: workgroup
+// i goes to XCD i % 8, and each XCD starts its workgroups in order), and the blocks of a head are numbered
+// consecutively in that order.  When one of them runs, every earlier head's blocks have started: those
+// finish without help from later workgroups and free their slots, which the remaining blocks of this head
+// are the next to take.  A head whose blocks fit one XCD's share of the device therefore never waits for a
+// workgroup that cannot start, however many heads the grid has -- and if that order were ever not kept,
+// the bounded wait reports it instead of hanging.
+// A (b, kv head) has at most 16 blocks up to 64k rows, at most peer_cap (32 in a workspace laid out for a
+// longer cache) beyond.  With the attention in the launch and a grid the device holds at once: the
+// smallest blocks that satisfy both -- more, lighter workgroups per head (measured at batch 1: 8k rows, 9
+// blocks of 1024: 11.3 us against 14.1 with 2 of 4096; 32k rows, 13 blocks of 2560: 14.1 against 15.5
+// with 9 of 4096; 40k rows, 16 of 2560: 14.7 against 16.0 with 10 of 4096; up to 64k rows more than 16
+// blocks measured slower again, and so did more than 8 rows per lane, which therefore only come in where
+// fewer, larger blocks are what it takes to keep the grid resident: batch 8 at 32k rows; 128k rows: 29
+// blocks of 4608 rows 24.6 us against 30.2 with 17 of 8192).  A grid the device cannot hold at once
+// (large batches) runs in rounds: then the fewest blocks per head, and the smallest rows per block that
+// give that few.  Without the attention (LRU table): 4096 rows where that fits (3072 in the case
+// described below), else 8192.
 template <typename T, int G, bool ATTEND>
 int pick_rows(int64_t n, int64_t heads, int peer_cap) {
     if (n < 1) n = 1;
     bool unknown = false;
     const int64_t most = n <= 16 * 4096 || peer_cap < 32 ? 16 : 32;
-    auto fits = [&](int spl) {
-        const int64_t rows = 512 * spl, blocks = (n + rows - 1) / rows;
+    auto blocks_of = [&](int spl) { return (n + 512 * spl - 1) / (512 * spl); };
+    // exists as a flavour, keeps a head within `most` blocks and within one XCD's share of the device
+    auto runs = [&](int spl) {
+        const int64_t blocks = blocks_of(spl);
         if (blocks > most) return false;
         const int slots = slots_rows<T, G, ATTEND>(spl, blocks > 16);
         if (slots == 0) unknown = true;
-        return heads * blocks <= slots;
+        return slots > 0 && blocks <= slots / SL_XCDS;
+    };
+    // ... and the whole grid is on the device at once (with the attention in the launch the blocks of
+    // a head share an XCD, heads c, c + 8, ... sit on XCD c: counted per XCD)
+    auto fits = [&](int spl) {
+        if (!runs(spl)) return false;
+        const int slots = slots_rows<T, G, ATTEND>(spl, blocks_of(spl) > 16);
+        if (ATTEND) return (heads + SL_XCDS - 1) / SL_XCDS * blocks_of(spl) <= slots / SL_XCDS;
+        return heads * blocks_of(spl) <= slots;
+    };
+    // a grid that runs in rounds: fewest blocks per head, then the smallest rows per block with that few
+    auto in_rounds = [&](const int *flavours, int count) {
+        int best = 0;
+        for (int i = 0; i < count; ++i) {
+            const int f = flavours[i];
+            if (!runs(f)) continue;
+            if (best == 0 || blocks_of(f) < blocks_of(best)) best = f;
+        }
+        return best;
     };
     int spl = 0;
-    if (g_fused_rows) spl = g_fused_rows % 512 == 0 && fits(g_fused_rows / 512) ? g_fused_rows / 512 : 0;
+    if (g_fused_rows) spl = g_fused_rows % 512 == 0 && runs(g_fused_rows / 512) ? g_fused_rows / 512 : 0;
     else if (ATTEND) {
         for (int f : FS_FLAVOURS)
             if (spl == 0 && fits(f)) spl = f;
@@ -346,9 +386,10 @@ int pick_rows(int64_t n, int64_t heads, int peer_cap) {
         // lane) that bring the launch down to one per compute unit win (batch 3 at 32k rows: 240
         // workgroups of 3584 rows 17.2 us against 312 of 2560 rows 17.9)
         const int64_t cus = sl_compute_units();
-        if (spl > 0 && spl < 8 && cus > 0 && heads * ((n + 512 * spl - 1) / (512 * spl)) > cus)
+        if (spl > 0 && spl < 8 && cus > 0 && heads * blocks_of(spl) > cus)
             for (int f = spl + 1; f <= 8; ++f)
-                if (fits(f) && heads * ((n + 512 * f - 1) / (512 * f)) <= cus) { spl = f; break; }
+                if (fits(f) && heads * blocks_of(f) <= cus) { spl = f; break; }
+        if (spl == 0) spl = in_rounds(FS_FLAVOURS, static_cast<int>(sizeof(FS_FLAVOURS) / sizeof(FS_FLAVOURS[0])));
     } else {
         // many workgroups per compute unit here (large batches): blocks of 3072 rows where they need
         // no more rounds of workgroups over the device than blocks of 4096 (C3: 768 workgroups, three
@@ -359,6 +400,8 @@ int pick_rows(int64_t n, int64_t heads, int peer_cap) {
             const int64_t w6 = heads * ((n + 3071) / 3072), w8 = heads * ((n + 4095) / 4096);
             if (cus > 0 && (w6 + cus - 1) / cus <= (w8 + cus - 1) / cus) spl = 6;
         }
+        static const int lru_flavours[] = {6, 8, 16};
+        if (spl == 0) spl = in_rounds(lru_flavours, 3);
     }
     return spl == 0 && unknown ? -1 : 512 * spl;
 }

@@ -35,6 +35,12 @@ struct hash_args {
     // launch's row is appended.  Later launches of the step read lengths from here, so that no launch
     // reads a length another workgroup of the same launch advances.
     int32_t *len_out;
+    // optional [B], with len_out: the rows the step keeps for a sequence that then holds n = len_out[b]
+    // rows, max(min(n, keep_min), n - int(n * keep_mask_out)), the product in double precision and
+    // truncated as Python's int() does (spotlight/modifiers/spotlight_generation.py:162-164)
+    int32_t *keep_out;
+    double keep_mask_out;
+    int keep_min;
     // optional rotary embedding of the inputs of every side before they are hashed (rotate_half
     // convention): inv_freq [d_in / 2] floats, position of batch entry b = rope_pos[b]
     const float *rope_inv_freq;

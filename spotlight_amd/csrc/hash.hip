@@ -206,8 +206,15 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
         }
     }
     // the step's row count per batch entry, for the launches that follow (head 0 of the last side)
-    if (a.len_out && sd.code_row && side_i == a.n_sides - 1 && h == 0 && tid < nb)
-        a.len_out[b_lo + tid] = (tid == 0 ? row0 : tid == 1 ? row1 : tid == 2 ? row2 : row3) + 1;
+    if (a.len_out && sd.code_row && side_i == a.n_sides - 1 && h == 0 && tid < nb) {
+        const int32_t n_now = (tid == 0 ? row0 : tid == 1 ? row1 : tid == 2 ? row2 : row3) + 1;
+        a.len_out[b_lo + tid] = n_now;
+        if (a.keep_out) {
+            const int32_t dropped = static_cast<int32_t>(static_cast<double>(n_now) * a.keep_mask_out);
+            const int32_t floor_k = n_now < a.keep_min ? n_now : a.keep_min;
+            a.keep_out[b_lo + tid] = n_now - dropped > floor_k ? n_now - dropped : floor_k;
+        }
+    }
     if (tid < HK_DIN) {
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) xs[rr][tid] = xrow[rr];

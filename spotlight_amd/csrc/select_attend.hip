@@ -45,11 +45,18 @@ __global__ __launch_bounds__(SA_THREADS) void select_attend_kernel(select_args s
     uint32_t cnt[SA_MAX_BPT], before[SA_MAX_BPT];
     const uint32_t mine = load_bins<SA_THREADS, SA_MAX_BPT, NG>(sa, bh, blk, cnt, before);
 
-    const int64_t n_b = tokens_of(sa, b);
-    const int k_eff = n_b < sa.k ? static_cast<int>(n_b) : sa.k;
+    int64_t n_b;
+    int k_eff;
+    rows_and_keep(sa, b, n_b, k_eff);
     int32_t *out = sa.idx + static_cast<int64_t>(bh) * sa.k;
     if (blk == 0)
         for (int i = k_eff + tid; i < sa.k; i += SA_THREADS) out[i] = -1;
+    if (n_b == 0) {   // no rows at all: nothing is kept, and the attention over nothing is zero
+        T *ob = static_cast<T *>(aa.out) + (static_cast<int64_t>(b) * aa.QH + static_cast<int64_t>(h) * G) * AT_D;
+        if (blk == 0)
+            for (int e = tid; e < G * AT_D; e += SA_THREADS) ob[e] = from_f32<T>(0.f);
+        return;
+    }
     if (static_cast<int64_t>(blk) * SA_BLOCK >= n_b) return;
     const int S = static_cast<int>((n_b + SA_BLOCK - 1) / SA_BLOCK);  // runs of this (b, kv head)
     const uint4 v = mask_run(raw, t0, n_b);

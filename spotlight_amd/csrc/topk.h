@@ -16,6 +16,7 @@ struct select_args {
     int n_blocks;             // row length of block_cnt
     int32_t *idx;             // [B, KH, k]
     const int32_t *seq_lens;  // optional
+    const int32_t *keep;      // optional [B] on the device: rows kept for sequence b this step, capped at k (needs seq_lens)
     int B, KH, k, n_bins, len_bias;
     int64_t n;
     int64_t stride_b, stride_n, stride_h;

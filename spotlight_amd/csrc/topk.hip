@@ -98,8 +98,9 @@ __global__ __launch_bounds__(TK_THREADS) void select_fused_kernel(select_args a)
     uint32_t cnt[MAX_BPT], before[MAX_BPT];
     const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, blk * (TK_BLOCK / a.hist_span), cnt, before);
 
-    const int64_t n_b = tokens_of(a, b);
-    const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
+    int64_t n_b;
+    int k_eff;
+    rows_and_keep(a, b, n_b, k_eff);
     int32_t *out = a.idx + static_cast<int64_t>(bh) * a.k;
     if (blk == 0)
         for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;
@@ -128,9 +129,10 @@ __global__ __launch_bounds__(TK_THREADS) void select_count_kernel(select_args a)
     const uint4 raw = load_run_raw<CONTIG>(a, sc, t0);
     uint32_t cnt[MAX_BPT], before[MAX_BPT];
     const uint32_t mine = load_bins<TK_THREADS, MAX_BPT, NG>(a, bh, 0, cnt, before);
-    const int64_t n_b = tokens_of(a, b);
+    int64_t n_b;
+    int k_eff;
+    rows_and_keep(a, b, n_b, k_eff);
     if (static_cast<int64_t>(blk) * TK_BLOCK >= n_b && blk > 0) return;
-    const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
     const uint4 v = mask_run(raw, t0, n_b);
     int thr, need;
     uint32_t tg_unused, te_unused;
@@ -153,8 +155,9 @@ __global__ __launch_bounds__(TK_THREADS) void select_compact_kernel(select_args 
     const int64_t t0 = static_cast<int64_t>(blk) * TK_BLOCK + tid * TK_RUN;
     const int16_t *sc = a.score + static_cast<int64_t>(b) * a.stride_b + static_cast<int64_t>(h) * a.stride_h;
     const uint4 raw = load_run_raw<CONTIG>(a, sc, t0);
-    const int64_t n_b = tokens_of(a, b);
-    const int k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
+    int64_t n_b;
+    int k_eff;
+    rows_and_keep(a, b, n_b, k_eff);
     int32_t *out = a.idx + static_cast<int64_t>(bh) * a.k;
     if (blk == 0)
         for (int i = k_eff + tid; i < a.k; i += TK_THREADS) out[i] = -1;

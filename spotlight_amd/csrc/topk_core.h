@@ -12,7 +12,27 @@ __device__ __forceinline__ int64_t tokens_of(const select_args &a, int b) {
         const int64_t l = static_cast<int64_t>(a.seq_lens[b]) + a.len_bias;
         n_b = l < n_b ? l : n_b;
     }
-    return n_b;
+    return n_b > 0 ? n_b : 0;   // a row count nobody has written yet (or a stale negative one) selects nothing
+}
+
+// Rows of sequence b (n_b) and how many of them are kept (k_eff): at most a.k, which is also the
+// row length of idx; at most the per-sequence budget the step's first launch left on the device
+// (a.keep, optional); at most the rows there are.  Both words are loaded before either is used
+// (an absent budget re-reads the row count and is ignored).
+__device__ __forceinline__ void rows_and_keep(const select_args &a, int b, int64_t &n_b, int &k_eff) {
+    if (!a.seq_lens) {
+        n_b = a.n > 0 ? a.n : 0;
+        k_eff = n_b < a.k ? static_cast<int>(n_b) : a.k;
+        return;
+    }
+    const int32_t l = a.seq_lens[b];
+    const int32_t kd = (a.keep ? a.keep : a.seq_lens)[b];
+    int64_t n = static_cast<int64_t>(l) + a.len_bias;
+    n = n < a.n ? n : a.n;
+    n_b = n > 0 ? n : 0;
+    int k = a.keep && kd < a.k ? kd : a.k;
+    k = k > 0 ? k : 0;
+    k_eff = n_b < k ? static_cast<int>(n_b) : k;
 }
 
 // ---- pieces shared by the select kernels ---------------------------------------

@@ -25,6 +25,11 @@ from . import kernel as K
 _L = _lib.load()
 
 
+class PeerWaitError(RuntimeError):
+    """A workgroup of the one-launch scorer + tail gave up waiting for the other blocks of its
+    (b, kv head): the indices and the attention output of that step are invalid."""
+
+
 @dataclass
 class HashWeights:
     """Per-head hash weights of one side (query or key).
@@ -78,7 +83,7 @@ class LayerDecodeState:
                  hash_q: HashWeights, hash_k: HashWeights, dtype=torch.bfloat16, device="cuda",
                  head_map: str = "blocked", lru_slots: int = 0, inputs=None, host_store: bool = False,
                  rope_theta: Optional[float] = None, rope_inv_freq: Optional[torch.Tensor] = None,
-                 codes_layout: str = "auto"):
+                 codes_layout: str = "auto", exclusive_device: bool = True):
         assert head_dim == 128, "the attention kernel covers head_dim 128"
         assert n_cap % 8 == 0, "n_cap must be a multiple of 8"
         assert hash_q.nbits == hash_k.nbits and hash_q.n_layers == hash_k.n_layers
@@ -97,6 +102,11 @@ class LayerDecodeState:
         # with an LRU table the launch ends at the selection).  "auto"
         # takes head-major whenever that launch covers the shape.  ``codes`` is always indexed
         # [b, row, kv head, word]; with head-major storage it is a strided view.
+        # The head-major step's workgroups wait for each other (bounded), which assumes that this launch
+        # has the device to itself: a caller whose other streams keep kernels running at the same time
+        # says so with exclusive_device=False and gets token-major codes, whose kernels never wait.
+        if codes_layout == "auto" and not exclusive_device:
+            codes_layout = "token"
         if codes_layout == "auto":
             # without an LRU table the launch also attends, one run per block of rows (up to 16 blocks per head,
             # 32 beyond 64k rows): keep <= 128 rows per block on average
@@ -249,13 +259,56 @@ class LayerDecodeState:
             _lib.check(_L.sl_workspace_init(self.ws.data_ptr(), self.ws.numel(),
                                             torch.cuda.current_stream().cuda_stream), "sl_workspace_init")
 
+    def error_word(self) -> Optional[torch.Tensor]:
+        """The device word (int32, shape [1]) a workgroup of the one-launch scorer + tail sets when it
+        gives up waiting for its peers; None with token-major codes, whose kernels never wait."""
+        off = _L.sl_decode_error_offset(C.byref(self.params))
+        if off == C.c_size_t(-1).value:
+            return None
+        return self.ws[off:off + 4].view(torch.int32)
+
     def peer_wait_failed(self) -> bool:
         """True if a workgroup of the one-launch scorer + tail ever gave up waiting for its peers (one
         device read; always False with token-major codes)."""
-        off = _L.sl_decode_error_offset(C.byref(self.params))
-        if off == C.c_size_t(-1).value:
-            return False
-        return bool(self.ws[off:off + 4].view(torch.int32).item())
+        w = self.error_word()
+        return False if w is None else bool(w.item())
+
+    def check_peer_wait(self, fallback: bool = True) -> None:
+        """Raises PeerWaitError if a bounded wait ran out since the last check (one device read, so
+        call it where the host synchronises anyway).  The word is cleared, and with ``fallback`` the
+        state moves to token-major codes first -- whose kernels never wait for each other -- so the
+        steps after the failed one are right whatever else keeps the device busy."""
+        if not self.peer_wait_failed():
+            return
+        self.error_word().zero_()
+        if fallback:
+            self.use_token_major()
+        raise PeerWaitError(
+            "a workgroup gave up waiting for the other blocks of its (batch entry, kv head): the last step's "
+            "indices and output are invalid (the device was probably shared with another stream's kernels)"
+            + ("; the state now uses token-major codes" if fallback else ""))
+
+    def use_token_major(self) -> None:
+        """Re-lay the key codes token-major and rebuild parameters and workspace for the three-launch
+        step.  Lengths, K/V, LRU table and the current budget are kept; a captured graph is dropped."""
+        if self.codes_layout == "token":
+            return
+        with torch.cuda.device(self.device):
+            torch.cuda.synchronize()
+            k_now, old = self.params.k, self.params
+            self._codes = self.codes.view(torch.int32).contiguous().view(torch.uint32)
+            self.codes = self._codes
+            self.codes_layout = "token"
+            self.params = self._make_params()
+            self.params.k = k_now
+            self.params.budget_on, self.params.budget_min_remain = old.budget_on, old.budget_min_remain
+            self.params.budget_mask_out = old.budget_mask_out
+            nbytes = _L.sl_decode_workspace_bytes(C.byref(self.params))
+            self.ws = torch.empty((nbytes,), dtype=torch.uint8, device=self.device)
+            _lib.check(_L.sl_workspace_init(self.ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream),
+                       "sl_workspace_init")
+            self.params.ws, self.params.ws_bytes = self.ws.data_ptr(), nbytes
+            self._graph = None
 
     def set_k(self, k: int) -> None:
         """Tokens kept per (b, kv head) from the next step on (at most the k given at
@@ -269,19 +322,39 @@ class LayerDecodeState:
         self.params.k = k
         self._graph = None
 
+    def set_budget(self, mask_out: Optional[float], min_remain: int = 0) -> None:
+        """Let the DEVICE evaluate the reference's budget rule every step
+        (spotlight_generation.py:162-164): a sequence that holds n rows after the append keeps
+        max(min(n, min_remain), n - int(n * mask_out)) of them, capped at ``current_k`` (the row
+        length of ``idx``; entries beyond the budget are -1).  Nothing on the host changes when the
+        budget does, so one captured graph serves a growing cache.  ``None`` switches the rule off."""
+        p = self.params
+        if mask_out is None:
+            p.budget_on = 0
+        else:
+            if not 0.0 <= mask_out <= 1.0 or min_remain < 0:
+                raise ValueError("mask_out must be in [0, 1] and min_remain >= 0")
+            p.budget_on, p.budget_min_remain, p.budget_mask_out = 1, int(min_remain), float(mask_out)
+        self._graph = None
+
     @property
     def current_k(self) -> int:
         return self.params.k
 
     def selected(self) -> torch.Tensor:
-        """int32 [B, KH, current_k]: the tokens the last step attended to, ascending."""
+        """int32 [B, KH, current_k]: the tokens the last step attended to, ascending; -1 beyond the
+        rows a sequence has, or beyond its budget.  Reads the device, so it also checks that no
+        bounded wait ran out (PeerWaitError)."""
+        self.check_peer_wait()
         k = self.params.k
         return self.idx.view(-1)[: self.B * self.KH * k].view(self.B, self.KH, k)
 
-    def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor) -> torch.Tensor:
+    def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, check: bool = False) -> torch.Tensor:
         """One decode step: q [B,QH,d], k_new/v_new [B,KH,d] (post-RoPE, or un-rotated when the
         state was built with ``rope_theta`` / ``rope_inv_freq``).
-        Returns the attention output [B,QH,d] (a buffer reused by the next step)."""
+        Returns the attention output [B,QH,d] (a buffer reused by the next step).  ``check``
+        synchronises and raises PeerWaitError if a bounded wait of this step ran out (debugging aid;
+        ``Spotlight.generate`` and ``selected`` check where they read the device anyway)."""
         with torch.cuda.device(self.device):
             if q is not self.q_in:
                 self.q_in.copy_(q)
@@ -291,6 +364,8 @@ class LayerDecodeState:
                 self.v_in.copy_(v_new)
             self._launch(self.host_len + 1)
         self.host_len += 1
+        if check:
+            self.check_peer_wait()
         return self.out
 
     def capture(self, steps_ahead: int) -> None:
@@ -312,3 +387,11 @@ class LayerDecodeState:
         self._graph_budget -= 1
         self.host_len += 1
         return self.out
+
+
+def any_peer_wait_failed(states) -> bool:
+    """One device read for many layer states: True if any of them has its error word set."""
+    words = [w for w in (st.error_word() for st in states) if w is not None]
+    if not words:
+        return False
+    return bool(torch.cat(words).any().item())

@@ -41,7 +41,7 @@ from typing import Optional
 import torch
 
 from .. import kernel as K
-from ..decode import HashWeights, LayerDecodeState
+from ..decode import HashWeights, LayerDecodeState, any_peer_wait_failed
 from ..modifier import Modifier
 
 
@@ -124,14 +124,24 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
 
 class SpotlightKV:
     """The per-layer cache handle threaded through the model in place of the
-    reference's ``(keys, vals)`` tuple."""
+    reference's ``(keys, vals)`` tuple.
+
+    A sparse layer's rows live in its ``LayerDecodeState``.  A dense layer keeps a plain K/V store,
+    head-major ``[B, KH, n_cap, d]`` (``keys`` / ``vals`` are ``[B, n_cap, KH, d]`` views of it), and
+    a device-side copy of its length, ``pos``: in *graph mode* (``Spotlight.generate`` replaying one
+    captured decode token) the forward takes every position from the device and never touches
+    ``length``, which the replay loop advances on the host."""
 
     def __init__(self, B, QH, KH, d, n_cap, dtype, device, sparse_state: Optional[LayerDecodeState]):
         self.B, self.QH, self.KH, self.d, self.n_cap = B, QH, KH, d, n_cap
         self.state = sparse_state
+        self.graph_mode = False
         if sparse_state is None:   # dense layer: plain K/V store
-            self.keys = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=device)
-            self.vals = torch.zeros((B, n_cap, KH, d), dtype=dtype, device=device)
+            self._k = torch.zeros((B, KH, n_cap, d), dtype=dtype, device=device)
+            self._v = torch.zeros((B, KH, n_cap, d), dtype=dtype, device=device)
+            self.keys, self.vals = self._k.permute(0, 2, 1, 3), self._v.permute(0, 2, 1, 3)
+            self.pos = torch.zeros((1,), dtype=torch.int64, device=device)
+            self.col = torch.arange(n_cap, device=device)
         else:
             self.keys, self.vals = sparse_state.keys, sparse_state.vals
         self.length = 0
@@ -140,9 +150,42 @@ class SpotlightKV:
         t = k.shape[1]
         if self.length + t > self.n_cap:
             raise RuntimeError(f"cache capacity {self.n_cap} exceeded")
-        K.cache_append(self.keys, k.contiguous(), start=self.length)
-        K.cache_append(self.vals, v.contiguous(), start=self.length)
+        self._k[:, :, self.length:self.length + t] = k.permute(0, 2, 1, 3)
+        self._v[:, :, self.length:self.length + t] = v.permute(0, 2, 1, 3)
         self.length += t
+
+    def enter_graph_mode(self):
+        if self.state is None:
+            self.pos.fill_(self.length)
+        self.graph_mode = True
+
+    def leave_graph_mode(self):
+        self.graph_mode = False
+
+    def advance(self, tokens: int):
+        """Host-side bookkeeping after ``tokens`` replays of the captured decode token (negative: rows
+        taken back; on the device too, where later steps simply overwrite them)."""
+        self.length += tokens
+        if self.state is not None:
+            self.state.host_len += tokens
+            if tokens < 0:
+                self.state.seq_lens.add_(tokens)
+        elif tokens < 0:
+            self.pos.add_(tokens)
+
+    def dense_decode_on_device(self, q, k, v):
+        """One new token of a dense layer with every position read from the device: q [B,1,QH,d],
+        k / v [B,1,KH,d], q and k already rotated at ``pos``.  The row goes into the store at ``pos``,
+        the attention runs over the whole capacity with the rows beyond ``pos`` masked, as two batched
+        matrix products per kv-head group (no K/V expansion), and ``pos`` advances."""
+        B, QH, KH, d = self.B, self.QH, self.KH, self.d
+        self._k.index_copy_(2, self.pos, k.permute(0, 2, 1, 3))
+        self._v.index_copy_(2, self.pos, v.permute(0, 2, 1, 3))
+        sc = torch.matmul(q.reshape(B, KH, QH // KH, d), self._k.transpose(2, 3)).float() * (d ** -0.5)
+        sc = sc.masked_fill((self.col > self.pos)[None, None, None, :], float("-inf"))
+        o = torch.matmul(torch.softmax(sc, dim=-1).to(q.dtype), self._v)
+        self.pos.add_(1)
+        return o.reshape(B, 1, QH, d)
 
 
 def _dense_attention(q, keys, vals):
@@ -185,11 +228,14 @@ def self_attn_forward(self, hidden_states: torch.Tensor, kv_cache=None):
 
     start = 0 if kv_cache is None else kv_cache.length
     theta = float(getattr(cfg, "rope_theta", 10000.0))
+    graph_mode = kv_cache is not None and kv_cache.graph_mode
+    if graph_mode and t != 1:
+        raise RuntimeError("graph mode covers one new token per call")
     # one new token of a sparse layer: the HIP step rotates q and the new key itself (at the
     # position it reads from the device-side length), so they are handed over un-rotated
     fused_rope = sparse and t == 1 and kv_cache is not None and kv_cache.length > 0
     if not fused_rope:
-        pos = torch.arange(start, start + t, device=dev)
+        pos = kv_cache.pos if graph_mode else torch.arange(start, start + t, device=dev)
         cos, sin = rope_tables(pos, d, theta, dtype)
         ques = apply_rope(ques, cos, sin)
         keys = apply_rope(keys, cos, sin)     # rotated once, here; stored post-RoPE
@@ -207,35 +253,49 @@ def self_attn_forward(self, hidden_states: torch.Tensor, kv_cache=None):
             hk = hq if per_qhead or KH == QH else self.hash_fn_k.hash_weights()
             k_cap = num_remain(n_cap, dk["mask_out"], dk["min_remain"])
             state = LayerDecodeState(B, QH, KHc, d, n_cap, k_cap, hq, hk,
-                                     dtype=dtype, device=dev, head_map="blocked", rope_theta=theta)
+                                     dtype=dtype, device=dev, head_map="blocked", rope_theta=theta,
+                                     exclusive_device=bool(dk.get("exclusive_device", True)))
+            # the budget (:162-164) is evaluated on the device from the length each step reads:
+            # nothing on the host changes when it grows, k_cap is only the row length of the index list
+            state.set_budget(float(dk["mask_out"]), int(dk["min_remain"]))
         kv_cache = SpotlightKV(B, QH, KHc, d, n_cap, dtype, dev, state)
 
     if t > 1 or not sparse or kv_cache.length == 0:
         # prefill (the draft is not used there, :145) and dense layers
-        if kv_cache.state is not None:
-            # rows, values and their codes go behind what is cached (chunked prefill included)
-            if kv_cache.length + t >= kv_cache.n_cap:
-                raise RuntimeError(f"cache capacity {kv_cache.n_cap} exceeded")
-            kv_cache.state.load_rows(keys.contiguous(), vals.contiguous(), start=kv_cache.length)
-            kv_cache.state.set_length(kv_cache.length + t)
-            kv_cache.length += t
+        if graph_mode:
+            out = kv_cache.dense_decode_on_device(ques, keys, vals)
         else:
-            kv_cache.append_dense(keys, vals)
-        n = kv_cache.length
-        out = _dense_attention(ques, kv_cache.keys[:, :n], kv_cache.vals[:, :n])
+            if kv_cache.state is not None:
+                # rows, values and their codes go behind what is cached (chunked prefill included)
+                if kv_cache.length + t >= kv_cache.n_cap:
+                    raise RuntimeError(f"cache capacity {kv_cache.n_cap} exceeded")
+                kv_cache.state.load_rows(keys.contiguous(), vals.contiguous(), start=kv_cache.length)
+                kv_cache.state.set_length(kv_cache.length + t)
+                kv_cache.length += t
+            else:
+                kv_cache.append_dense(keys, vals)
+            n = kv_cache.length
+            out = _dense_attention(ques, kv_cache.keys[:, :n], kv_cache.vals[:, :n])
+    elif graph_mode:
+        # the captured decode token: inputs into the step's own buffers, grid sized for the capacity,
+        # lengths and budget read from the device
+        st = kv_cache.state
+        st.q_in.copy_(ques[:, 0])
+        st.k_in.copy_(keys[:, 0])
+        st.v_in.copy_(vals[:, 0])
+        st._launch(st.n_cap)
+        out = st.out.unsqueeze(1)
     else:
         st = kv_cache.state
         n = kv_cache.length + 1
-        k = num_remain(n, dk["mask_out"], dk["min_remain"])
-        if k != st.current_k:
-            st.set_k(k)
         out = st.step(ques[:, 0].contiguous(), keys[:, 0].contiguous(), vals[:, 0].contiguous()).unsqueeze(1)
         kv_cache.length = n
         if dk.get("bench_mark", False):
             # benchmark mode (spotlight_evaluation.py:303-316): IoU of the selected rows
             # against the true top-k of q.k, per query head, averaged over the batch
             from ..iou import selection_iou
-            self.ratios = selection_iou(st.selected(), st.q_rot, kv_cache.keys[:, :n], k).mean(dim=0).tolist()
+            k = num_remain(n, dk["mask_out"], dk["min_remain"])
+            self.ratios = selection_iou(st.selected()[..., :k], st.q_rot, kv_cache.keys[:, :n], k).mean(dim=0).tolist()
 
     attn_output = self.o_proj(out.reshape(B, t, hidden))
     return attn_output, kv_cache
@@ -448,24 +508,109 @@ class Spotlight(Modifier):
     def generate(self, input_ids, max_new_tokens=128, eos_token_id=(2,)):
         """Greedy decoding (:470-495).  Batch 1 behaves exactly like the reference
         (stops at an eos token, which is not appended); a larger batch runs every
-        row for ``max_new_tokens`` steps."""
+        row for ``max_new_tokens`` steps.
+
+        On a GPU the decode token -- every layer, the final norm, ``lm_head`` and the argmax -- is
+        captured once as a HIP graph and replayed per token (``draft_kwargs["hip_graph"]``, default
+        on; off in benchmark mode, which reads the selection back every step): lengths, positions
+        and the budget all live on the device, so the graph stays valid while the cache grows."""
         if input_ids.ndim == 3:
             input_ids = input_ids.flatten(0, 1)
         device = next(iter(self.model.parameters())).device
         input_ids = input_ids.to(device)
-        output = self.model(input_ids=input_ids)
+        dk = self.conf["draft_kwargs"]
+        # the caches are sized by the first forward: make room for the tokens to come
+        need = input_ids.shape[1] + max_new_tokens + 8
+        given = dk.get("max_cache_len", None)
+        if int(given or 0) < need:
+            dk["max_cache_len"] = need
+        try:
+            output = self.model(input_ids=input_ids)
+        finally:
+            if given is None:
+                dk.pop("max_cache_len", None)
+            else:
+                dk["max_cache_len"] = given
         logits, kv_cache = output.logits, output.past_key_values
         new_tok = logits[:, -1:].argmax(dim=-1)
         new_ids = []
         single = input_ids.shape[0] == 1
+        use_graph = (bool(dk.get("hip_graph", True)) and device.type == "cuda" and not dk.get("bench_mark", False)
+                     and max_new_tokens > 2)
+        runner = None
+        unchecked = 0     # tokens decoded since the bounded waits were last looked at
+        states = [c.state for c in kv_cache if c is not None and c.state is not None]
         while len(new_ids) < max_new_tokens:
             if single and new_tok.ravel().item() in eos_token_id:
                 break
-            new_ids.append(new_tok)
-            output = self.model(input_ids=new_tok, kv_cache=kv_cache)
-            logits, kv_cache = output.logits, output.past_key_values
-            new_tok = logits[:, -1:].argmax(dim=-1)
+            new_ids.append(new_tok.clone())
+            if use_graph and runner is None and len(new_ids) == 2:
+                # (the first decoded token ran eagerly: lazy initialisations are behind us)
+                runner = _GraphedToken(self.model, kv_cache, new_tok)
+            if runner is not None:
+                new_tok = runner.replay(new_tok)
+            else:
+                output = self.model(input_ids=new_tok, kv_cache=kv_cache)
+                logits, kv_cache = output.logits, output.past_key_values
+                new_tok = logits[:, -1:].argmax(dim=-1)
+            unchecked += 1
+            # The head-major step's workgroups wait for each other (bounded): where the host reads the
+            # device anyway (batch 1: every token; otherwise every 16 tokens and at the end) the error
+            # words are looked at.  After a failure the affected tokens are taken back and decoded
+            # again, eagerly, on token-major codes, whose kernels never wait.
+            if states and (single or unchecked >= 16 or len(new_ids) == max_new_tokens):
+                if any_peer_wait_failed(states):
+                    if runner is not None:
+                        runner.close()
+                        runner, use_graph = None, False
+                    for st in states:
+                        if st.error_word() is not None:
+                            st.error_word().zero_()
+                        st.use_token_major()
+                    for c in kv_cache:
+                        c.advance(-unchecked)
+                    del new_ids[len(new_ids) - unchecked + 1:]
+                    new_tok = new_ids[-1]
+                    for _ in range(unchecked - 1):
+                        new_tok = self.model(input_ids=new_tok, kv_cache=kv_cache).logits[:, -1:].argmax(dim=-1)
+                        new_ids.append(new_tok)
+                    new_tok = self.model(input_ids=new_tok, kv_cache=kv_cache).logits[:, -1:].argmax(dim=-1)
+                unchecked = 0
+        if runner is not None:
+            runner.close()
         self.model.reset()
         if not new_ids:
             return input_ids
         return torch.cat([input_ids] + [t.to(input_ids.dtype) for t in new_ids], dim=-1)
+
+
+class _GraphedToken:
+    """One decode token of the whole model as a captured HIP graph: token ids in a fixed buffer, the
+    caches in graph mode (positions, lengths and budgets are read from the device), the next token
+    written back into the buffer by the graph itself."""
+
+    def __init__(self, model, kv_cache, tok):
+        self.kv_cache = kv_cache
+        self.tok = tok.clone()
+        for c in kv_cache:
+            c.enter_graph_mode()
+        self.graph = torch.cuda.CUDAGraph()
+        try:
+            with torch.cuda.graph(self.graph):
+                out = model(input_ids=self.tok, kv_cache=kv_cache)
+                self.tok.copy_(out.logits[:, -1:].argmax(dim=-1))
+        except Exception:
+            self.close()
+            raise
+
+    def replay(self, tok):
+        if tok is not self.tok:
+            self.tok.copy_(tok)
+        self.graph.replay()
+        for c in self.kv_cache:
+            c.advance(1)
+        return self.tok
+
+    def close(self):
+        for c in self.kv_cache:
+            c.leave_graph_mode()

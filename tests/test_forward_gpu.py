@@ -101,8 +101,11 @@ def test_pruned_decode_matches_the_reference_selection(gen, QH, KH):
         n = cache.length
         k = orc.num_remain(n, DK["mask_out"], DK["min_remain"])
         st = cache.state
-        assert st.current_k == k and ref_idx.shape[-1] == k
-        ours = st.selected().cpu().long()                              # [1, QH, k] (cache kept per query head)
+        # the budget is evaluated on the device: an index row is as long as the budget at capacity and
+        # holds -1 beyond this step's budget
+        full = st.selected().cpu().long()                              # [1, QH, k_cap] (cache kept per query head)
+        assert ref_idx.shape[-1] == k and (full[..., :k] >= 0).all() and (full[..., k:] == -1).all()
+        ours = full[..., :k]
         # reference scores per query head, recomputed from its cache
         keys_r, vals_r = ref_cache
         hid = x
@@ -168,5 +171,7 @@ def test_gqa_key_hash_mode_runs_batched(gen):
     assert n == 66 and cache.state.seq_lens.cpu().tolist() == [66] * 3
     k = orc.num_remain(n, 0.9, 8)
     idx = cache.state.selected().cpu().numpy()
-    assert idx.shape == (3, 2, k) and (np.diff(idx, axis=-1) > 0).all() and idx.max() < n
+    assert (idx[..., k:] == -1).all()          # beyond the budget the device evaluated for n rows
+    idx = idx[..., :k]
+    assert idx.shape == (3, 2, k) and (np.diff(idx, axis=-1) > 0).all() and idx.max() < n and idx.min() >= 0
     assert torch.isfinite(out.float()).all()

@@ -163,9 +163,10 @@ def test_pruned_generate_runs_the_sparse_step_and_matches_manual_loop(mods):
         out = m(input_ids=nxt, kv_cache=out.past_key_values)
         st = out.past_key_values[1].state
         n = 120 + step + 1
-        assert out.past_key_values[1].length == n and st.current_k == orc.num_remain(n, 0.9, 8)
+        k = orc.num_remain(n, 0.9, 8)
         idx = st.selected()
-        assert idx.shape[-1] == st.current_k and int(idx.max()) < n and int(idx.min()) >= 0
+        assert out.past_key_values[1].length == n and (idx[..., k:] == -1).all()   # the device's budget for n rows
+        assert int(idx[..., :k].max()) < n and int(idx[..., :k].min()) >= 0
     assert torch.equal(got[:, 120:], torch.cat(toks, dim=-1))
 
 
@@ -224,7 +225,9 @@ def test_linear_hashing_modifier(mods):
     assert got.shape == (1, 93)
     out = m(input_ids=ids.to(DEV))
     out = m(input_ids=got[:, 90:91], kv_cache=out.past_key_values)
-    assert out.past_key_values[1].state.current_k == orc.num_remain(91, 0.9, 8)
+    sel = out.past_key_values[1].state.selected()
+    k = orc.num_remain(91, 0.9, 8)
+    assert (sel[..., :k] >= 0).all() and (sel[..., k:] == -1).all()
     with pytest.raises(NotImplementedError):
         mods("upperbound-generation")
 
