@@ -33,36 +33,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
-CONFIGS = {
-    # name: B, QH, KH, n0, k, dtype, hash, lru slots, default layers, description
-    "c1": dict(B=1, QH=32, KH=32, n0=4096, k=410, dtype="f32", hash="linear", lru=0, layers=32,
-               desc="Llama-2-7B shape, fp32, linear 128x128 Gaussian hash, 90% pruned"),
-    "c2": dict(B=1, QH=32, KH=8, n0=32768, k=655, dtype="bf16", hash="mlp", lru=0, layers=32,
-               desc="Llama-3-8B GQA, bf16, 32k ctx, MLP 128-256-128 hash, 98% pruned"),
-    "c3": dict(B=16, QH=32, KH=8, n0=16384, k=328, dtype="bf16", hash="mlp", lru=1024, layers=32,
-               desc="Llama-3-8B GQA, bf16, batch 16 x 16k ctx, LRU resident buffer 1024, 98% pruned"),
-    "c4": dict(B=1, QH=40, KH=8, n0=131072, k=2622, dtype="bf16", hash="mlp", lru=0, layers=16,
-               desc="Qwen2.5-14B shape, bf16, 128k ctx, 98% pruned"),
-}
-
-
-def algorithmic_bytes(c, n):
-    """Bytes one step of one layer has to move, intermediates excluded."""
-    s = 4 if c["dtype"] == "f32" else 2
-    B, QH, KH, k, d, nbits = c["B"], c["QH"], c["KH"], c["k"], 128, 128
-    if c["hash"] == "mlp":
-        per_head = (128 * 256 + 256 + 256 * 128 + 128) * s
-        w = per_head * (QH + KH)
-    else:
-        w = 128 * 128 * s * (QH if KH == QH else QH + KH)
-    io_new = B * (QH + 2 * KH) * d * s                       # q, k_new, v_new read
-    append = B * KH * (nbits // 8 + 2 * d * s)               # code + K + V written
-    hash_b = w + io_new + append + B * QH * nbits // 8
-    score_b = B * n * KH * nbits // 8 + B * QH * nbits // 8  # codes streamed + q codes
-    attn_b = 2 * B * k * KH * d * s + 2 * B * QH * d * s     # selected K and V rows, q, out
-    lru_b = 0
-    return {"hash": hash_b, "score": score_b, "select": 0, "lru": lru_b, "attn": attn_b,
-            "step": w + B * QH * d * s + B * n * KH * nbits // 8 + 2 * B * k * KH * d * s + B * QH * d * s + append}
+from spotlight_amd.workloads import CONFIGS, E2EModel, algorithmic_bytes, build_layers  # noqa: E402
 
 
 def main():
@@ -86,6 +57,9 @@ def main():
                     help="only measure what the step's launches cost by themselves (near-empty kernels on the step's grids)")
     ap.add_argument("--codes-layout", default="auto", choices=["auto", "token", "head"],
                     help="key-code layout: head-major runs scorer, selection and attention as one launch")
+    ap.add_argument("--via-modifier", action="store_true",
+                    help="c5 only: drive a Llama-3-8B-shaped nn.Module through get_modifier('spotlight-generation-hip') "
+                         "and Spotlight.generate (the drop-in path) instead of the hand-written decode token")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-breakdown", action="store_true")
     args = ap.parse_args()
@@ -99,7 +73,7 @@ def main():
     from spotlight_amd import _lib, decode, kernel
 
     if args.config == "c5":
-        return run_e2e(args)
+        return run_e2e_modifier(args) if args.via_modifier else run_e2e(args)
     for kv in args.tune:
         key, val = kv.split("=")
         _lib.check(_lib.load().sl_tune(key.encode(), int(val)), f"sl_tune({kv})")
@@ -124,7 +98,8 @@ def main():
 
     # the timed region is whole tokens (one graph replay = one token = L steps): the number of steps asked
     # for is rounded to whole tokens, at least one, and the warm-up covers every layer at least once
-    tokens_timed = max(1, round(steps / L))
+    # (at least 8 tokens whatever --steps says: one replay alone is a sub-millisecond sample)
+    tokens_timed = max(8, round(steps / L))
     tokens_warm = max(1, math.ceil(warmup / L))
     steps_timed, steps_warm = tokens_timed * L, tokens_warm * L
     tokens = tokens_warm + tokens_timed + 4 + 64   # cache growth incl. the breakdown passes
@@ -136,8 +111,6 @@ def main():
         print(json.dumps({"config": args.config, "latency_floor": latency_floor(dev, c, L, n0 + tokens, reps=64, one_launch_tail=head)}), flush=True)
         return
 
-    cpu_gen = torch.Generator()
-    cpu_gen.manual_seed(0)
     gpu_gen = torch.Generator(device=dev)
     gpu_gen.manual_seed(0)
 
@@ -148,31 +121,8 @@ def main():
     cur = [torch.empty((1, L, B, h, d), device=dev, dtype=dtype) for h in (QH, KH, KH)]
     tok = torch.zeros((1,), dtype=torch.int64, device=dev)
 
-    layers = []
-    for li in range(L):
-        if c["hash"] == "mlp":
-            hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, dev, cpu_gen)
-            hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, dev, cpu_gen)
-        else:
-            hq = decode.HashWeights.random_linear(QH, 128, 128, dtype, dev, cpu_gen)
-            hk = hq if KH == QH else decode.HashWeights.random_linear(KH, 128, 128, dtype, dev, cpu_gen)
-        st = decode.LayerDecodeState(B, QH, KH, d, n_cap, k, hq, hk, dtype=dtype, device=dev,
-                                     lru_slots=c["lru"], inputs=tuple(t[0, li] for t in cur),
-                                     host_store=args.host_store, codes_layout=args.codes_layout)
-        # prefill in slabs to bound the transient memory of hashing
-        st.seq_lens.zero_()
-        slab = max(1, (1 << 22) // (B * KH))
-        for s0 in range(0, n0, slab):
-            s1 = min(n0, s0 + slab)
-            kk = torch.randn((B, s1 - s0, KH, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
-            vv = torch.randn((B, s1 - s0, KH, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
-            st.keys[:, s0:s1] = kk      # (a device-to-host copy with --host-store)
-            st.vals[:, s0:s1] = vv
-            st.hash_k.hash_rows(kk, out=st.codes[:, s0:s1])
-        st.seq_lens.fill_(n0)
-        st.host_len = n0
-        layers.append(st)
-    torch.cuda.synchronize()
+    layers = build_layers(c, L, n_cap, dev, codes_layout=args.codes_layout, host_store=args.host_store,
+                          inputs=[tuple(t[0, li] for t in cur) for li in range(L)])
 
     def token_body(n_max):
         for i in range(3):
@@ -190,20 +140,34 @@ def main():
     n_max = n0 + tokens
     token_graph = capture(lambda: token_body(n_max))
 
-    for _ in range(tokens_warm):
+    # cold figure: the very first replay on freshly built layer states (kernel code, weights, codes and
+    # translation entries all come from memory for the first time); it is also the first warm-up token
+    torch.cuda.synchronize()
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    token_graph.replay()
+    c1.record()
+    torch.cuda.synchronize()
+    cold_first_token_us = c0.elapsed_time(c1) * 1e3 / L
+    for _ in range(tokens_warm - 1):
         token_graph.replay()
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(tokens_timed + 1)]
     t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(tokens_timed):
+    marks[0].record()
+    for i in range(tokens_timed):
         token_graph.replay()
-    ev1.record()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    gpu_ms = ev0.elapsed_time(ev1)
+    gpu_ms = marks[0].elapsed_time(marks[-1])
+    per_token_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 / L for i in range(tokens_timed))
     ms_per_step = wall_ms / steps_timed
     us_per_step = ms_per_step * 1e3
+    # a bounded wait that ran out would have produced wrong rows silently: no figure is reported then
+    failed = [i for i, st in enumerate(layers) if st.peer_wait_failed()]
+    if failed:
+        raise RuntimeError(f"bounded peer wait ran out in layers {failed}: the timed steps are invalid")
     n_mid = n0 + tokens_warm + tokens_timed / 2
     ab = algorithmic_bytes(c, n_mid)
     for st in layers:   # the graph advanced the lengths on the device; keep the host-side bound in step
@@ -289,6 +253,9 @@ def main():
         cpu_baseline = cpu_leg(layers[0], c, budget_s=12.0)
         cpu_reference_form = cpu_leg_reference_form(layers[0], c, budget_s=12.0)
 
+    failed = [i for i, st in enumerate(layers) if st.peer_wait_failed()]
+    if failed:
+        raise RuntimeError(f"bounded peer wait ran out in layers {failed} during the per-kernel passes")
     step_gbps = ab["step"] / us_per_step / 1e3
     out = {
         "metric": "sparse-decode us/step/layer (Llama-3-8B GQA, 32k ctx)" if args.config == "c2"
@@ -304,6 +271,9 @@ def main():
                    "layers_rotated": L,
                    "graph": f"one HIP graph per token ({L} steps); {tokens_timed} replays timed after {tokens_warm} warm-up replays"},
         "gpu_event_ms_per_step": round(gpu_ms / steps_timed, 6),
+        "us_per_step_median_token": round(per_token_us[len(per_token_us) // 2], 3),
+        "us_per_step_min_token": round(per_token_us[0], 3), "us_per_step_max_token": round(per_token_us[-1], 3),
+        "cold_first_token_us": round(cold_first_token_us, 3),
         "hbm_gbps": round(step_gbps, 1), "hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(ab["step"]),
         "tokens_per_s": round(B / (ms_per_step * 1e-3 * L), 2), "tokens_per_s_layers": L,
@@ -313,153 +283,6 @@ def main():
         "value_over_floor": round(us_per_step / floor["launches_with_one_load_us"], 2) if floor else None,
     }
     print(json.dumps(out), flush=True)
-
-
-class E2EModel:
-    """Random-init Llama-shaped decoder (RMSNorm, rotary GQA attention, SiLU-gated MLP; defaults are
-    Llama-3-8B's dims: hidden 4096, 32 q / 8 kv heads of 128, MLP 14336, vocab 128256, rope theta 5e5)
-    whose layers in ``fix_layers`` attend densely and whose other layers run the sparse HIP step
-    (k rows kept, MLP hash 128-256-128 per query head and per kv head).  It stands for the loop of
-    the reference's ``generate`` (spotlight_generation.py:470-495) with dense layers 0-1
-    (config/llama3-8b-spotlight-generation.json).  ``step_body`` is one decoded token for the
-    whole batch and is capturable as one HIP graph: positions and lengths live on the device, and
-    the sparse step rotates q and the new key itself."""
-
-    def __init__(self, L=32, B=4, n0=32768, n_cap=None, k=655, fix_layers=(0, 1), hidden=4096, inter=14336,
-                 vocab=128256, QH=32, KH=8, theta=5e5, seed=0):
-        import torch
-
-        from spotlight_amd import decode
-        self.dev = dev = torch.device("cuda:0")
-        self.dt = dt = torch.bfloat16
-        self.L, self.B, self.n0, self.k, self.QH, self.KH, self.d = L, B, n0, k, QH, KH, 128
-        self.hidden, self.vocab, self.theta = hidden, vocab, theta
-        self.n_cap = n_cap or (n0 + 1024 + 7) // 8 * 8
-        d = self.d
-        g = torch.Generator(device=dev)
-        g.manual_seed(seed)
-        cg = torch.Generator()
-        cg.manual_seed(seed)
-        self.g = g
-        rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * 0.02).to(dt)
-        self.embed, self.lm_head = rnd(vocab, hidden), rnd(vocab, hidden)
-        self.layers = []
-        for li in range(L):
-            w = dict(wq=rnd(QH * d, hidden), wk=rnd(KH * d, hidden), wv=rnd(KH * d, hidden), wo=rnd(hidden, QH * d),
-                     wg=rnd(inter, hidden), wu=rnd(inter, hidden), wd=rnd(hidden, inter),
-                     n1=torch.ones(hidden, device=dev, dtype=dt), n2=torch.ones(hidden, device=dev, dtype=dt))
-            if li in fix_layers:
-                w["kc"] = torch.zeros((B, KH, self.n_cap, d), device=dev, dtype=dt)   # head-major: read in place
-                w["vc"] = torch.zeros((B, KH, self.n_cap, d), device=dev, dtype=dt)
-            else:
-                hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dt, dev, cg)
-                hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dt, dev, cg)
-                w["st"] = decode.LayerDecodeState(B, QH, KH, d, self.n_cap, k, hq, hk, dtype=dt, device=dev,
-                                                  rope_theta=theta)
-            self.layers.append(w)
-        self.norm_f = torch.ones(hidden, device=dev, dtype=dt)
-        self.inv_freq = 1.0 / (theta ** (torch.arange(0, d, 2, device=dev, dtype=torch.float32) / d))
-        self.tok = torch.zeros((B,), dtype=torch.int64, device=dev)
-        self.logits = torch.zeros((B, vocab), dtype=torch.float32, device=dev)   # of the last decoded token
-        self.pos = torch.full((1,), n0, dtype=torch.int64, device=dev)
-        self.col = torch.arange(self.n_cap, device=dev)
-        self.sparse = [w["st"] for w in self.layers if "st" in w]
-
-    def rms(self, x, w):
-        import torch
-        xf = x.float()
-        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).to(self.dt) * w
-
-    def rope(self, x, pos):   # x [..., t, H, d], pos [t] (device)
-        import torch
-        d = self.d
-        ang = pos.float()[:, None] * self.inv_freq[None, :]
-        emb = torch.cat((ang, ang), dim=-1)
-        cos, sin = emb.cos().to(self.dt)[:, None, :], emb.sin().to(self.dt)[:, None, :]
-        rot = torch.cat((-x[..., d // 2:], x[..., : d // 2]), dim=-1)
-        return x * cos + rot * sin
-
-    def mlp(self, w, h):
-        import torch.nn.functional as F
-        return (F.silu(h @ w["wg"].T) * (h @ w["wu"].T)) @ w["wd"].T
-
-    def prefill(self):
-        """Dense causal attention in every layer (the draft is not used there), one sequence at a
-        time; sparse layers also get the codes of their keys.  Returns the seconds it took."""
-        import torch
-        import torch.nn.functional as F
-
-        from spotlight_amd import kernel
-        B, n0, QH, KH, d, dev = self.B, self.n0, self.QH, self.KH, self.d, self.dev
-        t_pre = time.perf_counter()
-        pos0 = torch.arange(n0, device=dev)
-        with torch.no_grad():
-            for b in range(B):
-                ids = torch.randint(0, self.vocab, (n0,), generator=self.g, device=dev)
-                x = self.embed[ids]                                                   # [n0, hidden]
-                for w in self.layers:
-                    h = self.rms(x, w["n1"])
-                    q = self.rope((h @ w["wq"].T).view(n0, QH, d), pos0)
-                    kk = self.rope((h @ w["wk"].T).view(n0, KH, d), pos0)
-                    vv = (h @ w["wv"].T).view(n0, KH, d)
-                    o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], kk.transpose(0, 1)[None],
-                                                       vv.transpose(0, 1)[None], is_causal=True, enable_gqa=True)
-                    x = x + o[0].transpose(0, 1).reshape(n0, QH * d) @ w["wo"].T
-                    x = x + self.mlp(w, self.rms(x, w["n2"]))
-                    if "st" in w:
-                        st = w["st"]
-                        st.keys[b, :n0] = kk
-                        st.vals[b, :n0] = vv
-                        st.hash_k.hash_rows(kk[None], out=st.codes[b:b + 1, :n0])
-                    else:
-                        w["kc"][b, :, :n0] = kk.transpose(0, 1)
-                        w["vc"][b, :, :n0] = vv.transpose(0, 1)
-                self.tok[b] = (self.rms(x[-1:], self.norm_f) @ self.lm_head.T).float().argmax(dim=-1)[0]
-                del x, h, q, kk, vv, o
-            for st in self.sparse:
-                st.set_length(n0)
-        torch.cuda.synchronize()
-        return time.perf_counter() - t_pre
-
-    def step_body(self):
-        import torch
-        B, QH, KH, d, dt = self.B, self.QH, self.KH, self.d, self.dt
-        x = self.embed[self.tok]                                                       # [B, hidden]
-        for w in self.layers:
-            h = self.rms(x, w["n1"])
-            q = (h @ w["wq"].T).view(B, QH, d)
-            kk = (h @ w["wk"].T).view(B, KH, d)
-            vv = (h @ w["wv"].T).view(B, KH, d)
-            if "st" in w:
-                st = w["st"]          # un-rotated q and k: the step rotates them at its own position
-                st.q_in.copy_(q)
-                st.k_in.copy_(kk)
-                st.v_in.copy_(vv)
-                st._launch(self.n_cap)
-                o = st.out.reshape(B, QH * d)
-            else:
-                q = self.rope(q[:, None], self.pos)[:, 0]
-                kk = self.rope(kk[:, None], self.pos)[:, 0]
-                w["kc"].index_copy_(2, self.pos, kk[:, :, None])
-                w["vc"].index_copy_(2, self.pos, vv[:, :, None])
-                # dense decode attention as two batched GEMMs per kv head group (the G query heads of
-                # a kv head are the G rows of the left operand: no K/V expansion, K and V read once)
-                sc = torch.matmul(q.view(B, KH, QH // KH, d), w["kc"].transpose(2, 3)).float() * (d ** -0.5)
-                sc = sc.masked_fill((self.col > self.pos)[None, None, None, :], float("-inf"))
-                o = torch.matmul(torch.softmax(sc, dim=-1).to(dt), w["vc"]).reshape(B, QH * d)
-            x = x + o @ w["wo"].T
-            x = x + self.mlp(w, self.rms(x, w["n2"]))
-        self.logits.copy_((self.rms(x, self.norm_f) @ self.lm_head.T).float())
-        self.tok.copy_(self.logits.argmax(dim=-1))
-        self.pos.add_(1)
-
-    def rewind(self, tokens, tok):
-        """Undo the last ``tokens`` decoded tokens: positions and lengths go back, the input token is
-        restored.  Rows beyond the lengths are simply overwritten by the next steps."""
-        self.pos.sub_(tokens)
-        self.tok.copy_(tok)
-        for st in self.sparse:
-            st.seq_lens.sub_(tokens)
 
 
 def run_e2e(args):
@@ -525,6 +348,49 @@ def run_e2e(args):
         "roofline": None, "cpu_baseline": None,
     }
     print(json.dumps(out), flush=True)
+
+
+def run_e2e_modifier(args):
+    """c5 through the drop-in path: a random-init Llama-3-8B-shaped nn.Module patched by
+    get_modifier('spotlight-generation-hip') (layers 0-1 dense, per-kv-head key hash, MLP 128-256-128, 98 %
+    pruned with the budget rule evaluated on the device), batch 4, 32768-token prompt prefilled densely by the
+    patched forward, then ``Spotlight.generate``: first decoded token eagerly, the rest as replays of the one
+    HIP graph ``generate`` captures.  `value` is decoded tokens per second over the decode part of ``generate``
+    (its own clock, bracketed by device synchronisation)."""
+    import torch
+
+    from spotlight_amd.modifiers import get_modifier
+    from spotlight_amd.workloads import llama_shaped
+
+    L = args.layers or 32
+    steps = args.steps if args.steps is not None else 64
+    B, n0 = args.batch or 4, args.context or 32768
+    conf = {"draft_kwargs": {"enable": True, "fix_layers": [0, 1], "mask_out": 0.98, "bench_mark": False, "min_remain": 20,
+                             "num_mlp_layers": 2, "mlp_dims": "[128,256,128]", "mlp_residue": False, "gqa_key_hash": True,
+                             "record_timing": True}}
+    base = llama_shaped(L=L)
+    _, cls = get_modifier("spotlight-generation-hip")
+    m = cls(base, None, None, conf).eval()
+    ids = torch.randint(0, base.config.vocab_size, (B, n0), generator=torch.Generator().manual_seed(0))
+    out = m.generate(ids, max_new_tokens=steps, eos_token_id=[-1])
+    assert out.shape == (B, n0 + steps)
+    t = m.timing
+    ms_per_token = t["graph_decode_s"] * 1e3 / max(1, t["graph_tokens"]) if t["graph_tokens"] else t["decode_s"] * 1e3 / steps
+    res = {
+        "metric": "e2e greedy decode tokens/s through the patched modifier (random-init Llama-3-8B, batch 4, 32k prompt)",
+        "value": round(B / (ms_per_token * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 1,
+        "ms_per_step": round(ms_per_token, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "c5 via the modifier: get_modifier('spotlight-generation-hip') -> Spotlight.generate on a "
+                               "random-init Llama-3-8B-shaped nn.Module, batch 4, 32768-token dense prefill, greedy decode, "
+                               "layers 0-1 dense, 98 % pruned (budget rule on the device)",
+                   "layers": L, "batch": B, "context": n0,
+                   "graph": "generate() captures the decode token once and replays it"},
+        "prefill_s": round(t["prefill_s"], 2), "first_decode_token_ms": round(t["eager_decode_s"] * 1e3 / max(1, t["eager_tokens"]), 3),
+        "graph_tokens": t["graph_tokens"], "eager_tokens": t["eager_tokens"], "capture_s": round(t["capture_s"], 3),
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(res), flush=True)
 
 
 _STAGES_NO_ADVANCE = 1 | 2 | 4 | 16     # hash, score, select, attention launched as stages: lengths do not advance

@@ -59,8 +59,10 @@ int sl_version(void);
  * workgroup instead of 4 (default 128);
  * "attn_mfma": 1 puts the q.K products of the attention on the matrix cores
  * (16-bit inputs; default 0: packed dot products and a lane butterfly);
- * "fused_rows": rows per block of the step over head-major codes (4096, 8192;
- * 0 = 4096 while all blocks are resident at once, the default);
+ * "fused_rows": rows per block of the step over head-major codes: 512 x {1 .. 12,
+ * 14, 16}, the sizes that exist as kernels (other values are refused; a size that
+ * would give a head more blocks than it may have makes sl_decode_step return
+ * SL_ERR_UNSUPPORTED); 0 = by shape, the default;
  * "fused_spin_limit", "fused_phantom_peer": for testing the bounded wait of that
  * step -- polls before a workgroup gives up (0 = the default, 2^22) and 1 = every
  * head also waits for a block that does not exist, so that each workgroup gives
@@ -358,6 +360,19 @@ int sl_decode_stages(const sl_decode_params *p, int stages, void *stream);
  * graph of such launches with the decode step's grids measures what the
  * launches themselves cost on a machine, i.e. the floor under the step. */
 int sl_probe_launch(int blocks, int threads, const uint32_t *table, uint32_t *sink, int chain, void *stream);
+
+/* Measurement aid (no counterpart in the reference).  A library built with
+ * -DSL_PHASE_STAMPS (`python -m spotlight_amd.build --stamps`) has lane 0 of the
+ * first SL_STAMP_WGS workgroups of a launch store the 100 MHz wall clock at up
+ * to SL_STAMP_SLOTS numbered points of the kernel; this call copies the table
+ * of `kernel` ("hash", "fused", "attn", "select_attend", "lru") to HOST memory
+ * `host` (SL_STAMP_WGS * SL_STAMP_SLOTS words: slot i of workgroup w at
+ * w * SL_STAMP_SLOTS + i, 0 = not reached) after the caller has synchronised,
+ * and with `clear` zeroes the device table.  The product library carries no
+ * stamps and returns SL_ERR_UNSUPPORTED. */
+#define SL_STAMP_WGS 4096
+#define SL_STAMP_SLOTS 24
+int sl_phase_stamps(const char *kernel, unsigned long long *host, size_t host_words, int clear);
 
 /* Zero-fills a workspace with a kernel (safe inside a captured HIP graph). */
 int sl_workspace_init(void *ws, size_t ws_bytes, void *stream);

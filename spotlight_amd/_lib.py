@@ -14,6 +14,7 @@ LIB_PATH = os.environ.get("SPOTLIGHT_HIP_LIB") or os.path.join(_HERE, "libspotli
 
 SL_F32, SL_BF16, SL_F16 = 0, 1, 2
 SL_HEADMAP_INTERLEAVED, SL_HEADMAP_BLOCKED = 0, 1
+STAMP_WGS, STAMP_SLOTS = 4096, 24
 STAGE_HASH, STAGE_SCORE, STAGE_SELECT, STAGE_LRU, STAGE_ATTN, STAGE_ALL = 1, 2, 4, 8, 16, 31
 
 c_void_p, c_int, c_int64, c_size_t, c_float, c_uint32 = (
@@ -71,6 +72,7 @@ SIGNATURES = {
     "sl_decode_stages": (c_int, [C.POINTER(DecodeParams), c_int, c_void_p]),
     "sl_probe_launch": (c_int, [c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "sl_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
+    "sl_phase_stamps": (c_int, [C.c_char_p, c_void_p, c_size_t, c_int]),
 }
 
 _lib = None

@@ -31,14 +31,21 @@ def _hipcc() -> str:
     return exe
 
 
-def build_library(verbose: bool = True, jobs: int = 4) -> str:
+STAMPS_LIB_PATH = os.path.join(HERE, "libspotlight_hip_stamps.so")
+
+
+def build_library(verbose: bool = True, jobs: int = 4, stamps: bool = False) -> str:
     """Compile every kernel source and link the shared library.  Always
-    recompiles; returns the path of the built library."""
+    recompiles; returns the path of the built library.  ``stamps``: the
+    measurement build (-DSL_PHASE_STAMPS, csrc/phase_stamps.h) as a second
+    library, libspotlight_hip_stamps.so, which SPOTLIGHT_HIP_LIB selects."""
     from concurrent.futures import ThreadPoolExecutor
 
     hipcc = _hipcc()
-    objdir = os.path.join(CSRC, "build")
+    objdir = os.path.join(CSRC, "build_stamps" if stamps else "build")
     os.makedirs(objdir, exist_ok=True)
+    flags = HIPCC_FLAGS + (["-DSL_PHASE_STAMPS"] if stamps else [])
+    lib_path = STAMPS_LIB_PATH if stamps else LIB_PATH
 
     def run(cmd) -> None:
         if verbose:
@@ -54,16 +61,15 @@ def build_library(verbose: bool = True, jobs: int = 4) -> str:
 
     def compile_one(src: str) -> str:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        run([hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        run([hipcc, *flags, "-c", os.path.join(CSRC, src), "-o", obj])
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(compile_one, SOURCES))
-    run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", LIB_PATH])
-    return LIB_PATH
+    run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", lib_path])
+    return lib_path
 
 
 if __name__ == "__main__":
-    build_library()
-    print(LIB_PATH)
+    print(build_library(stamps="--stamps" in sys.argv[1:], jobs=8 if "-j8" in sys.argv[1:] else 4))
     sys.exit(0)

@@ -6,6 +6,8 @@
 // consecutive ranks, one workgroup of 4 waves per run; the run's row numbers
 // are fetched into LDS in one go and the shared body (attn_core.h) does the
 // rest.
+#define SL_TS_NAME "attn"
+#include "phase_stamps.h"
 #include "attn_core.h"
 
 #include <string.h>

@@ -28,6 +28,9 @@
 // result does not depend on arrival order.
 #pragma once
 #include "attn.h"
+#ifndef SL_TS
+#include "phase_stamps.h"
+#endif
 
 constexpr int AT_D = 128;
 constexpr int AT_PART = AT_D + 2;    // acc[128], m, l
@@ -256,6 +259,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
 #pragma unroll
     for (int g = 0; g < G; ++g) { lsum[g] = 0.f; acc[g][0] = 0.f; acc[g][1] = 0.f; }
 
+    SL_TS(10);  // attention: query slices requested
     for (int base = 0; base < n_rows; base += CH) {
         // every load of the chunk first: U key slices for the score phase, RW value
         // pairs for the accumulation phase (an absent or skipped row re-reads row 0
@@ -304,6 +308,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         // scores.  Dot flavour: partial dot products of this lane's slice, then the butterfly: ONE
         // score per lane.  Matrix-core flavour: four instructions leave FOUR scores per lane (head
         // lane % 16 of the rows 4 (lane / 16) .. + 3 of the wave's tile).
+        if (base == 0) SL_TS(11);  // first chunk: K / V loads issued
         constexpr int NS = MF ? 4 : 1;
         float sc[NS];
         bool valid[NS];
@@ -352,6 +357,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             const float wm = head_max<U>(sc[0]);
             if (lane < 16 && u_l == 0) sh.wmax[wave][g_l] = wm;
         }
+        if (base == 0) SL_TS(12);  // first chunk: scores done (K rows arrived)
         __syncthreads();
         float m_new[GP];
 #pragma unroll
@@ -376,6 +382,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
 
         // values: rescale what earlier chunks left (exp(-inf) = 0 on the first), then
         // accumulate this wave's rows of the chunk
+        if (base == 0) SL_TS(13);  // first chunk: probabilities in LDS
         if (base > 0) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
@@ -407,6 +414,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         if (base + CH < n_rows) __syncthreads();  // the next chunk rewrites wmax and p
     }
 
+    SL_TS(14);  // all chunks done
     // the waves' tiles meet in LDS
 #pragma unroll
     for (int g = 0; g < G; ++g) *reinterpret_cast<float2 *>(&sh.acc[wave][g][lane * 2]) = make_float2(acc[g][0], acc[g][1]);
@@ -426,6 +434,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         sh.L[tid] = L;
     }
 
+    SL_TS(15);
     const int bh = b * a.KH + h;
     T *ob = static_cast<T *>(a.out) + (static_cast<int64_t>(b) * a.QH + static_cast<int64_t>(h) * G) * AT_D;
     float *part_out = a.part + (static_cast<int64_t>(bh) * AT_PART_SPLITS + split) * G * AT_PART;
@@ -453,10 +462,13 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         st_agent(part_out + tid * AT_PART + AT_D, sh.M[tid]);
         st_agent(part_out + tid * AT_PART + AT_D + 1, sh.L[tid]);
     }
+    SL_TS(16);  // partials stored
     publish_wait();
     __syncthreads();
+    SL_TS(17);  // ... and acknowledged
     if (tid == 0) sh.last = arrive_last(&a.counter[bh], static_cast<uint32_t>(S));
     __syncthreads();
+    SL_TS(18);  // ticket taken
     if (!sh.last) return;
 
     // merge the S runs by log-sum-exp.  All loads are issued together: the runs'
@@ -476,6 +488,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             pa[i][sp] = e < G * AT_D ? v : 0.f;
         }
     }
+    SL_TS(19);  // merge: loads of all runs issued
     static_assert(MAXS == 16 || MAXS == 32, "the runs of a head fit one 16-lane row, or half a wave");
     for (int g = wave; g < G; g += NW) {
         // lanes 0 .. MAXS - 1 hold one run each: with 16 runs the reductions stay inside a 16-lane row
@@ -503,6 +516,7 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
             ob[e] = from_f32<T>(L > 0.f ? O / L : 0.f);
         }
     }
+    SL_TS(20);  // merged output stored
     if (a.peer_flag && tid < S) st_agent(&a.peer_flag[static_cast<int64_t>(bh) * a.peer_flag_stride + tid], 0u);
     if (tid == 0) {
         st_agent(&a.counter[bh], 0u);

@@ -1,6 +1,9 @@
 // (d) cache append, row gather and the LRU resident table.
 #include "lru.h"
 
+#define SL_TS_NAME "lru"
+#include "phase_stamps.h"
+
 namespace {
 
 // ---- append ---------------------------------------------------------------------
@@ -75,6 +78,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
     __shared__ uint32_t s_digit, s_remaining;
     __shared__ int s_new_in, s_new_pos;
 
+    SL_TS(0);   // start
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.KH, h = blockIdx.x % a.KH;
     const int C = a.C, k = a.k;
@@ -144,6 +148,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
     }
     __syncthreads();
 
+    SL_TS(1);   // wanted rows classified against the map, misses listed
     if (M > 0) {
         const int SPT = (C + LRU_THREADS - 1) / LRU_THREADS;
         uint32_t key[4];
@@ -199,6 +204,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
             prefix |= s_digit << shift;
             remaining = s_remaining;
         }
+        SL_TS(2);   // radix passes done: threshold stamp known
         const uint32_t thr = prefix, need_eq = remaining;
         uint32_t lt = 0, eq = 0;
 #pragma unroll
@@ -227,6 +233,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
         }
         __syncthreads();
 
+        SL_TS(3);   // victims listed
         // fetch the missed rows from the full store into their slots: LRU_CP 16-byte
         // chunks of K and of V per lane are in flight at once, and they are issued
         // before the bookkeeping below, which does not depend on them
@@ -268,6 +275,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
     }
 #undef LRU_ISSUE
 #undef LRU_RETIRE
+    SL_TS(4);   // table updated
     if (tid == 0 && a.stats) {
         a.stats[bh * 2] += static_cast<uint32_t>(n_wanted - M);
         a.stats[bh * 2 + 1] += static_cast<uint32_t>(M);

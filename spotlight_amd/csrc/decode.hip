@@ -23,6 +23,17 @@
 #include "select_attend.h"
 #include "topk.h"
 
+#ifdef SL_PHASE_STAMPS
+#include <vector>
+typedef int (*sl_ts_reader)(unsigned long long *host, int clear);
+namespace {
+struct ts_entry { const char *name; sl_ts_reader fn; };
+std::vector<ts_entry> &ts_registry() { static std::vector<ts_entry> r; return r; }
+}  // namespace
+// called by every instrumented translation unit while the library is loaded
+void sl_ts_register(const char *name, sl_ts_reader fn) { ts_registry().push_back({name, fn}); }
+#endif
+
 namespace {
 
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint4 *p, size_t n16, uint8_t *tail, size_t n_tail) {
@@ -112,6 +123,27 @@ extern "C" int sl_probe_launch(int blocks, int threads, const uint32_t *table, u
     if (chain > 0) SL_REQUIRE(table && sink, SL_ERR_NULL);
     probe_kernel<<<dim3(blocks), dim3(threads), 0, static_cast<hipStream_t>(stream)>>>(table, sink, chain);
     return sl_check_launch();
+}
+
+extern "C" int sl_phase_stamps(const char *kernel, unsigned long long *host, size_t host_words, int clear) {
+#ifdef SL_PHASE_STAMPS
+    SL_REQUIRE(kernel && host, SL_ERR_NULL);
+    SL_REQUIRE(host_words >= static_cast<size_t>(SL_STAMP_WGS) * SL_STAMP_SLOTS, SL_ERR_WORKSPACE);
+    // several translation units may carry one name (one per element type and group size): the one
+    // whose kernel ran is the one with stamps in its table
+    int found = 0;
+    for (const ts_entry &e : ts_registry()) {
+        if (strcmp(e.name, kernel) != 0) continue;
+        found = 1;
+        if (e.fn(host, clear) != 0) return SL_ERR_LAUNCH;
+        for (size_t i = 0; i < static_cast<size_t>(SL_STAMP_WGS) * SL_STAMP_SLOTS; ++i)
+            if (host[i]) return SL_OK;
+    }
+    return found ? SL_OK : SL_ERR_SHAPE;
+#else
+    (void)kernel; (void)host; (void)host_words; (void)clear;
+    return SL_ERR_UNSUPPORTED;
+#endif
 }
 
 extern "C" int sl_host_device_pointer(void *host_ptr, void **device_ptr) {

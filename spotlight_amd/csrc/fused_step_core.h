@@ -5,6 +5,10 @@
 
 #include <atomic>
 
+#ifndef SL_TS_NAME
+#define SL_TS_NAME "fused"
+#endif
+#include "phase_stamps.h"
 #include "attn_core.h"
 #include "topk_core.h"
 
@@ -35,6 +39,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     __shared__ int32_t s_list[FS_BLOCK];
     __shared__ attn_shared<ATTEND ? G : 1, FS_NW> sh;
 
+    SL_TS(0);   // start
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // With the attention in the launch the blocks of a (b, kv head) share an XCD (see xcd_unmap): they swap
     // histograms and merge their runs (measured: 0.5 - 0.7 us per step at batch 1 - 3).  Without it, and for
@@ -90,6 +95,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     if (tid == 0) { s_range[0] = NB; s_range[1] = -1; }
     __syncthreads();
 
+    SL_TS(1);   // row count known, LDS histogram cleared
     // scores: matching bits summed over the G query heads; -1 marks a row past the end
     int sc[FS_SLOTS];
     int s_lo = NB, s_hi = -1;
@@ -108,6 +114,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
             s_hi = sc[j] > s_hi ? sc[j] : s_hi;
         }
     }
+    SL_TS(2);   // codes arrived, scores counted
     // the block's score range: only these bins of its histogram can be non-empty
     s_lo = wave_min_i32(s_lo);
     s_hi = wave_max_i32(s_hi);
@@ -126,6 +133,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
         for (int e = tid; e < NB; e += FS_THREADS) st_agent(peers + blk * FS_NB_PAD + e, s_hist[e]);
         publish_wait();
         __syncthreads();
+        SL_TS(3);   // own histogram published and acknowledged
         // the flag carries the block's range: bit 31 = published, bits 12.. = hi, bits 0..11 = lo
         if (tid == 0) st_agent(flags + blk, 0x80000000u | (static_cast<uint32_t>(hi) << 12) | static_cast<uint32_t>(lo));
         if (wave == 0) {
@@ -142,6 +150,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
             if (lane == 0) { s_range[0] = all_lo; s_range[1] = all_hi; }
         }
         __syncthreads();
+        SL_TS(4);   // every peer's flag seen
         lo = s_range[0]; hi = s_range[1];
     }
     const int n_ranks = hi - lo + 1;
@@ -177,10 +186,12 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
         }
     }
 
+    SL_TS(5);   // peers' bins read and summed
     int thr, need;
     uint32_t tg, te;
     find_threshold<FS_THREADS, FS_MAX_BPT>(hi, n_ranks, cnt, before, mine, k_eff, s_wave, s_tn, thr, need, tg, te);
 
+    SL_TS(6);   // threshold known
     // placement in row order (wave, slot, lane): ballots give every kept row its position
     uint32_t mgt_lo[FS_SLOTS], mgt_hi[FS_SLOTS], meq_lo[FS_SLOTS], meq_hi[FS_SLOTS];
     uint32_t wave_gt = 0, wave_eq = 0;
@@ -222,6 +233,7 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
 
     // the list goes out with coalesced stores; the attention then runs over it
     __syncthreads();
+    SL_TS(7);   // kept rows listed in LDS
     for (int i = tid; i < n_kept; i += FS_THREADS) out[first + i] = s_list[i];
     if constexpr (ATTEND) {
         attend_rows_and_merge<T, G, FS_NW, false, false, MAXS>(aa, b, h, blk, S, s_list, n_kept, sh);

@@ -24,6 +24,9 @@
 // (after the matmul, after the bias add, after SiLU, after the residual add).
 #include "hash.h"
 
+#define SL_TS_NAME "hash"
+#include "phase_stamps.h"
+
 #include <string.h>
 
 namespace {
@@ -92,6 +95,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     __shared__ float sub[R * HK_THREADS];
     __shared__ float hidl[R][D_HID];
 
+    SL_TS(0);   // start
     const int tid = threadIdx.x;
     const int hh = blockIdx.x;
     const int side_i = (a.n_sides > 1 && hh >= a.side[0].H) ? 1 : 0;
@@ -215,12 +219,14 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
             a.keep_out[b_lo + tid] = n_now - dropped > floor_k ? n_now - dropped : floor_k;
         }
     }
+    SL_TS(1);   // inputs arrived (and rotated)
     if (tid < HK_DIN) {
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) xs[rr][tid] = xrow[rr];
     }
     __syncthreads();
 
+    SL_TS(2);
     // first projection
     {
         float acc[R][8];
@@ -245,8 +251,10 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
         }
     }
     __syncthreads();
+    SL_TS(3);   // first projection's partial sums in LDS: its weights have arrived
     float v1[R];
     fold_columns<D_HID, R>(red, sub, v1);
+    SL_TS(4);
     if (tid < D_HID) {
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
@@ -261,6 +269,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
         for (int rr = 0; rr < R; ++rr) pre[rr] = v1[rr];
     } else {
         __syncthreads();
+        SL_TS(5);
         // second projection
         {
             float acc[R][8];
@@ -285,7 +294,9 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
             }
         }
         __syncthreads();
+        SL_TS(6);   // second projection's partial sums in LDS
         fold_columns<HK_NBITS, R>(red, sub, pre);
+        SL_TS(7);
         if (tid < HK_NBITS) {
 #pragma unroll
             for (int rr = 0; rr < R; ++rr)
@@ -306,6 +317,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
         }
     }
 
+    SL_TS(8);   // codes stored
     // cache append of the new K and V rows (loaded at the top)
     if (cp_live) {
         const int64_t dst_off = static_cast<int64_t>(cp_b) * sd.copy_dst_stride_b +

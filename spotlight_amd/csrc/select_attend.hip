@@ -13,6 +13,8 @@
 // Used for up to 16 blocks (64k tokens) and up to 1024 score bins.
 #include "select_attend.h"
 
+#define SL_TS_NAME "select_attend"
+#include "phase_stamps.h"
 #include "attn_core.h"
 #include "topk_core.h"
 

@@ -35,6 +35,7 @@ from __future__ import annotations
 
 import json
 import math
+import time
 import types
 from typing import Optional
 
@@ -524,6 +525,17 @@ class Spotlight(Modifier):
         given = dk.get("max_cache_len", None)
         if int(given or 0) < need:
             dk["max_cache_len"] = need
+        # draft_kwargs["record_timing"]: leave the seconds spent in prefill, in eagerly decoded tokens, in the
+        # capture and in replayed tokens in ``self.timing`` (each phase bracketed by a device synchronisation)
+        rec = bool(dk.get("record_timing", False)) and device.type == "cuda"
+        timing = dict(prefill_s=0.0, eager_decode_s=0.0, eager_tokens=0, capture_s=0.0, graph_decode_s=0.0, graph_tokens=0)
+
+        def clock():
+            if rec:
+                torch.cuda.synchronize(device)
+            return time.perf_counter()
+
+        t_mark = clock()
         try:
             output = self.model(input_ids=input_ids)
         finally:
@@ -533,6 +545,7 @@ class Spotlight(Modifier):
                 dk["max_cache_len"] = given
         logits, kv_cache = output.logits, output.past_key_values
         new_tok = logits[:, -1:].argmax(dim=-1)
+        timing["prefill_s"] = clock() - t_mark
         new_ids = []
         single = input_ids.shape[0] == 1
         use_graph = (bool(dk.get("hip_graph", True)) and device.type == "cuda" and not dk.get("bench_mark", False)
@@ -546,13 +559,20 @@ class Spotlight(Modifier):
             new_ids.append(new_tok.clone())
             if use_graph and runner is None and len(new_ids) == 2:
                 # (the first decoded token ran eagerly: lazy initialisations are behind us)
+                t_mark = clock()
                 runner = _GraphedToken(self.model, kv_cache, new_tok)
+                timing["capture_s"] = clock() - t_mark
+            t_mark = clock() if rec and (runner is None or timing["graph_tokens"] == 0) else t_mark
             if runner is not None:
                 new_tok = runner.replay(new_tok)
+                timing["graph_tokens"] += 1
             else:
                 output = self.model(input_ids=new_tok, kv_cache=kv_cache)
                 logits, kv_cache = output.logits, output.past_key_values
                 new_tok = logits[:, -1:].argmax(dim=-1)
+                if rec:
+                    timing["eager_decode_s"] += clock() - t_mark
+                timing["eager_tokens"] += 1
             unchecked += 1
             # The head-major step's workgroups wait for each other (bounded): where the host reads the
             # device anyway (batch 1: every token; otherwise every 16 tokens and at the end) the error
@@ -577,7 +597,11 @@ class Spotlight(Modifier):
                     new_tok = self.model(input_ids=new_tok, kv_cache=kv_cache).logits[:, -1:].argmax(dim=-1)
                 unchecked = 0
         if runner is not None:
+            if rec:    # the replays are timed as one stretch: nothing synchronises between them but the checks above
+                timing["graph_decode_s"] = clock() - t_mark
             runner.close()
+        timing["decode_s"] = timing["eager_decode_s"] + timing["graph_decode_s"]
+        self.timing = timing
         self.model.reset()
         if not new_ids:
             return input_ids

@@ -13,8 +13,8 @@ pytestmark = pytest.mark.gpu
 def model():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
-    import bench
-    m = bench.E2EModel(L=4, B=4, n0=32768, k=655, fix_layers=(0,), seed=3)
+    from spotlight_amd.workloads import E2EModel
+    m = E2EModel(L=4, B=4, n0=32768, k=655, fix_layers=(0,), seed=3)
     m.prefill()
     return m
 
