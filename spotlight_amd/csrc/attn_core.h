@@ -292,14 +292,26 @@ __device__ __forceinline__ void attend_rows_and_merge(const attn_args &a, int b,
         }
         pair_raw<T> vs[RW];
         int vrow[RW], vsrc[RW];
+        // the RW rows this wave accumulates: lane j reads the number of row j (ONE trip to LDS for the
+        // wave, not one per row -- each would be waited for before the row's load could be issued) and
+        // the loop below takes it from that lane
+        static_assert(RW <= 64, "one lane per row of the wave's share of a chunk");
+        int r_lane, s_lane = -1;
+        {
+            const int ri = base + wave + NW * (lane < RW ? lane : 0);
+            const bool in = lane < RW && ri < n_rows;
+            r_lane = s_row[in ? ri : 0];
+            if constexpr (FETCH) s_lane = s_src[in ? ri : 0];
+            r_lane = in ? r_lane : -1;
+            s_lane = in && r_lane >= 0 ? s_lane : -1;
+        }
 #pragma unroll
         for (int j = 0; j < RW; ++j) {
-            const int ri = base + wave + NW * j;
-            int r = ri < n_rows ? s_row[ri] : -1;
-            int sr = FETCH && ri < n_rows && r >= 0 ? s_src[ri] : -1;
-            vrow[j] = __builtin_amdgcn_readfirstlane(r);
-            vsrc[j] = __builtin_amdgcn_readfirstlane(sr);
-            r = __builtin_amdgcn_readfirstlane(r >= 0 ? r : 0);  // the same row for the whole wave
+            int r = __builtin_amdgcn_readlane(r_lane, j);
+            const int sr = FETCH ? __builtin_amdgcn_readlane(s_lane, j) : -1;
+            vrow[j] = r;
+            vsrc[j] = sr;
+            r = r >= 0 ? r : 0;  // the same row for the whole wave
             const T *p = vb + static_cast<int64_t>(r) * a.kv_stride_n;
             if constexpr (FETCH) p = vsrc[j] >= 0 ? svb + static_cast<int64_t>(vsrc[j]) * a.src_stride_n : p;
             vs[j] = load_pair<T>(p);

@@ -528,7 +528,7 @@ class Spotlight(Modifier):
         # draft_kwargs["record_timing"]: leave the seconds spent in prefill, in eagerly decoded tokens, in the
         # capture and in replayed tokens in ``self.timing`` (each phase bracketed by a device synchronisation)
         rec = bool(dk.get("record_timing", False)) and device.type == "cuda"
-        timing = dict(prefill_s=0.0, eager_decode_s=0.0, eager_tokens=0, capture_s=0.0, graph_decode_s=0.0, graph_tokens=0)
+        timing = dict(prefill_s=0.0, eager_decode_s=0.0, eager_tokens=0, capture_s=0.0, graph_decode_s=0.0, graph_tokens=0, recoveries=0)
 
         def clock():
             if rec:
@@ -557,7 +557,7 @@ class Spotlight(Modifier):
             if single and new_tok.ravel().item() in eos_token_id:
                 break
             new_ids.append(new_tok.clone())
-            if use_graph and runner is None and len(new_ids) == 2:
+            if use_graph and runner is None and len(new_ids) >= 2:
                 # (the first decoded token ran eagerly: lazy initialisations are behind us)
                 t_mark = clock()
                 runner = _GraphedToken(self.model, kv_cache, new_tok)
@@ -580,9 +580,10 @@ class Spotlight(Modifier):
             # again, eagerly, on token-major codes, whose kernels never wait.
             if states and (single or unchecked >= 16 or len(new_ids) == max_new_tokens):
                 if any_peer_wait_failed(states):
-                    if runner is not None:
+                    timing["recoveries"] += 1
+                    if runner is not None:    # (captured again below, over token-major codes)
                         runner.close()
-                        runner, use_graph = None, False
+                        runner = None
                     for st in states:
                         if st.error_word() is not None:
                             st.error_word().zero_()

@@ -610,3 +610,195 @@ def test_rotation_uses_each_sequence_s_own_position(env):
     assert (k_rows.float() - orc.apply_rope(kn, lens, theta).float()).abs().max() <= 2e-2
     assert torch.equal(st.q_rot[1].cpu(), q[1])            # position 0: the identity
     assert st.seq_lens.tolist() == [l + 1 for l in lens]
+
+
+@pytest.mark.parametrize("layout", ["head", "token"])
+def test_budget_rule_on_the_device_survives_graph_replay_across_a_change_of_k(env, layout):
+    """The budget max(min(n, min_remain), n - int(n * mask_out)) (spotlight_generation.py:162-164) is
+    evaluated on the device from the length each step reads, so ONE captured graph keeps matching the
+    oracle while k changes (here: 0.9 of the rows dropped, k grows every few tokens), in a ragged batch
+    whose sequences have different lengths and therefore different budgets."""
+    decode, kernel = env
+    dtype = torch.bfloat16
+    B, QH, KH, n0 = 2, 8, 2, 1195
+    mask_out, min_remain = 0.9, 20
+    n_cap = 1280
+    k_cap = orc.num_remain(n_cap, mask_out, min_remain)
+    st = _make_state(decode, _gen(310), B, QH, KH, n0, n_cap, k_cap, dtype, codes_layout=layout)
+    st.seq_lens.copy_(torch.tensor([n0, n0 - 333], dtype=torch.int32))      # second sequence is shorter
+    st.set_budget(mask_out, min_remain)
+    g = _gen(311)
+    st.capture(steps_ahead=40)
+    ks = set()
+    for step in range(30):
+        q, kn, vn = (torch.randn(B, h, 128, generator=g).to(dtype) for h in (QH, KH, KH))
+        st.q_in.copy_(q.to(DEV)); st.k_in.copy_(kn.to(DEV)); st.v_in.copy_(vn.to(DEV))
+        out = st.replay().float().cpu().numpy()
+        idx = st.selected().cpu().numpy()
+        assert idx.shape == (B, KH, k_cap)
+        q_code = kernel.hash_mlp_pack(q.to(DEV), st.hash_q.w1, st.hash_q.b1, st.hash_q.w2, st.hash_q.b2).cpu().numpy()[:, None]
+        for b, n in enumerate([n0 + step + 1, n0 - 333 + step + 1]):
+            k = orc.num_remain(n, mask_out, min_remain)
+            ks.add(k)
+            score = orc.hamming_score_u32(q_code[b:b + 1], st.codes[b:b + 1, :n].cpu().numpy(), "blocked")
+            want = orc.topk_stable(score, k)
+            np.testing.assert_array_equal(idx[b:b + 1, :, :k], want, err_msg=f"step {step} sequence {b} k {k}")
+            assert (idx[b, :, k:] == -1).all()
+            ref = orc.sparse_attention(q[b:b + 1].float().numpy(), st.keys[b:b + 1, :n].float().cpu().numpy(),
+                                       st.vals[b:b + 1, :n].float().cpu().numpy(), want)
+            assert np.abs(out[b:b + 1] - ref).max() <= TOL[dtype], (step, b)
+    assert len(ks) >= 6          # the budget did change under the one graph, several times
+    assert st.seq_lens.cpu().tolist() == [n0 + 30, n0 - 333 + 30]
+
+
+def test_budget_rule_matches_python_for_awkward_products(env):
+    """int(n * mask_out) truncates a double-precision product; the device must land on the same side
+    of every integer boundary as Python does (mask_out values whose products sit just below / above
+    an integer), and below min_remain rows everything is kept."""
+    decode, kernel = env
+    dtype = torch.float32
+    B, QH, KH = 1, 2, 2
+    for mask_out, min_remain in [(0.98, 20), (0.7, 5), (0.1, 3), (0.29, 1), (0.57, 0), (1.0, 4), (0.0, 2)]:
+        n_cap = 256
+        k_cap = n_cap
+        st = _make_state(decode, _gen(int(mask_out * 100) + 3), B, QH, KH, 1, n_cap, k_cap, dtype, codes_layout="token")
+        st.set_budget(mask_out, min_remain)
+        g = _gen(5)
+        for step in range(120):
+            q, kn, vn = (torch.randn(B, h, 128, generator=g).to(dtype) for h in (QH, KH, KH))
+            st.step(q.to(DEV), kn.to(DEV), vn.to(DEV))
+            n = 2 + step
+            k = orc.num_remain(n, mask_out, min_remain)
+            kept = (st.idx[0, 0] >= 0).sum().item()
+            assert kept == min(k, n), (mask_out, min_remain, n, kept, k)
+
+
+@pytest.mark.parametrize("lru", [0, 256])
+def test_a_bounded_wait_that_ran_out_is_raised_and_the_state_falls_back_to_token_major(env, lru):
+    """What the product path does with the error word: check_peer_wait() (called by selected() and by
+    Spotlight.generate where they read the device anyway) raises PeerWaitError, clears the word and
+    re-lays the codes token-major, whose kernels never wait; lengths, rows, LRU table and budget are
+    kept and the next steps are right.  The failure is forced from the host (a peer that does not
+    exist, a short poll limit): every kernel still finishes normally."""
+    decode, kernel = env
+    from spotlight_amd import _lib
+    L = _lib.load()
+    dtype = torch.bfloat16
+    B, QH, KH, n0, k = 1, 8, 2, 9000, 100
+    st = _make_state(decode, _gen(185), B, QH, KH, n0, (n0 + 64 + 7) // 8 * 8, k, dtype, lru=lru, codes_layout="head")
+    g = _gen(186)
+    fresh = lambda: tuple(torch.randn(B, h, 128, generator=g).to(dtype) for h in (QH, KH, KH))
+    q, kn, vn = fresh()
+    st.step(q.to(DEV), kn.to(DEV), vn.to(DEV), check=True)       # healthy: no raise
+    _lib.check(L.sl_tune(b"fused_spin_limit", 64), "sl_tune")
+    _lib.check(L.sl_tune(b"fused_phantom_peer", 1), "sl_tune")
+    try:
+        q, kn, vn = fresh()
+        with pytest.raises(decode.PeerWaitError):
+            st.step(q.to(DEV), kn.to(DEV), vn.to(DEV), check=True)
+    finally:
+        _lib.check(L.sl_tune(b"fused_spin_limit", 0), "sl_tune")
+        _lib.check(L.sl_tune(b"fused_phantom_peer", 0), "sl_tune")
+    assert st.codes_layout == "token" and not st.peer_wait_failed()
+    assert st.seq_lens.cpu().tolist() == [n0 + 2] * B               # the failed step did append its row
+    for step in range(2):
+        q, kn, vn = fresh()
+        out = st.step(q.to(DEV), kn.to(DEV), vn.to(DEV), check=True).clone()
+        if lru == 0:
+            _check_step(kernel, st, q, kn, vn, out, n0 + 2 + step, dtype)
+        else:
+            assert st.seq_lens.cpu().tolist() == [n0 + 3 + step] * B
+            idx = st.selected().cpu().numpy()
+            q_code = kernel.hash_mlp_pack(q.to(DEV), st.hash_q.w1, st.hash_q.b1, st.hash_q.w2, st.hash_q.b2).cpu().numpy()[:, None]
+            n = n0 + 3 + step
+            want = orc.topk_stable(orc.hamming_score_u32(q_code, st.codes[:, :n].cpu().numpy(), "blocked"), k)
+            np.testing.assert_array_equal(idx, want)
+    # selected() is the other place that looks: a word set behind its back is raised there
+    st2 = _make_state(decode, _gen(187), B, QH, KH, n0, (n0 + 64 + 7) // 8 * 8, k, dtype, lru=lru, codes_layout="head")
+    st2.error_word().fill_(1)
+    with pytest.raises(decode.PeerWaitError):
+        st2.selected()
+    assert st2.codes_layout == "token"
+
+
+def test_head_major_grids_larger_than_the_device_run_in_rounds(env):
+    """Batches whose grid the device cannot hold at once (hundreds of (b, kv head) pairs times several
+    blocks) still run the one-launch step: the blocks of a head are numbered consecutively in start
+    order, so a head never waits for a workgroup that cannot start.  Indices must equal the
+    token-major step's, outputs agree to rounding, and no bounded wait may run out."""
+    decode, kernel = env
+    from spotlight_amd import _lib
+    L = _lib.load()
+    dtype = torch.bfloat16
+    try:
+        for case, (B, KH, G, n0, k, rows, lru) in enumerate([(64, 8, 4, 1500, 30, 512, 0), (48, 8, 1, 3000, 64, 1024, 0),
+                                                             (32, 8, 4, 2500, 50, 0, 0), (64, 4, 2, 5000, 100, 1024, 0),
+                                                             (64, 8, 4, 7000, 60, 3072, 128), (40, 8, 5, 2000, 40, 512, 0)]):
+            QH = KH * G
+            n_cap = (n0 + 16 + 7) // 8 * 8
+            cg = torch.Generator().manual_seed(900 + case)
+            g = torch.Generator(device=DEV).manual_seed(900 + case)
+            hq = decode.HashWeights.random_mlp(QH, [128, 256, 128], dtype, DEV, cg)
+            hk = decode.HashWeights.random_mlp(KH, [128, 256, 128], dtype, DEV, cg)
+            kk = torch.randn((B, n0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+            vv = torch.randn((B, n0, KH, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype)
+            head, token = (decode.LayerDecodeState(B, QH, KH, 128, n_cap, k, hq, hk, dtype=dtype, device=DEV, lru_slots=lru,
+                                                   codes_layout=layout) for layout in ("head", "token"))
+            head.prefill(kk, vv)
+            token.prefill(kk, vv)
+            _lib.check(L.sl_tune(b"fused_rows", rows), "sl_tune")
+            for step in range(2):
+                q, kn, vn = (torch.randn((B, h, 128), generator=g, device=DEV, dtype=torch.float32).to(dtype) for h in (QH, KH, KH))
+                a = head.step(q, kn, vn).float().clone()
+                b = token.step(q, kn, vn).float().clone()
+                assert not head.peer_wait_failed(), (case, step)
+                assert torch.equal(head.idx, token.idx), (case, step)
+                assert (a - b).abs().max().item() <= TOL[dtype], (case, step)
+    finally:
+        _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
+
+
+def test_seeded_inputs_end_to_end_against_the_oracle_s_own_codes(env):
+    """ONE seeded input through both pipelines from the raw vectors on: the oracle hashes the query and
+    every key itself (fp64 pre-activations -> sign -> pack), scores, selects and attends; the GPU does
+    the same from the same vectors (prompt keys through the many-rows hash, the decoded token through
+    the step).  Where no pre-activation lies within the margin of zero -- asserted for these seeds, so
+    the comparison is not vacuous -- the codes, and with them the kept indices, must be identical; else
+    the count is reported and the comparison falls back to the codes the GPU holds."""
+    decode, kernel = env
+    dtype, margin = torch.float32, 1e-4
+    B, QH, KH, n0, k = 2, 4, 2, 300, 40
+    g = _gen(300)
+
+    def mk(H):
+        w = [torch.randn(H, 128, 256, generator=g) * 0.5, torch.randn(H, 256, 128, generator=g) * 0.5]
+        b = [torch.randn(H, 256, generator=g) * 0.5, torch.randn(H, 128, generator=g) * 0.5]
+        return w, b
+    (wq, bq), (wk, bk) = mk(QH), mk(KH)
+    keys_all = torch.randn(B, n0 + 1, KH, 128, generator=g)
+    q = torch.randn(B, QH, 128, generator=g)
+    vals_all = torch.randn(B, n0 + 1, KH, 128, generator=g)
+    as_np = lambda w, b: [(w[0].numpy(), b[0].numpy()), (w[1].numpy(), b[1].numpy())]
+    pre_k = orc.mlp_hash(keys_all.reshape(B * (n0 + 1), KH, 128).numpy(), as_np(wk, bk), False)
+    pre_q = orc.mlp_hash(q.numpy(), as_np(wq, bq), False)
+    inside = int((np.abs(pre_k) < margin).sum() + (np.abs(pre_q) < margin).sum())
+    codes_o = orc.pack_sign_u32(pre_k).reshape(B, n0 + 1, KH, 4)
+    hq = decode.HashWeights(wq[0].to(DEV), bq[0].to(DEV), wq[1].to(DEV), bq[1].to(DEV))
+    hk = decode.HashWeights(wk[0].to(DEV), bk[0].to(DEV), wk[1].to(DEV), bk[1].to(DEV))
+    for layout in ("head", "token"):
+        st = decode.LayerDecodeState(B, QH, KH, 128, 320, k, hq, hk, dtype=dtype, device=DEV, codes_layout=layout)
+        st.prefill(keys_all[:, :n0].to(DEV), vals_all[:, :n0].to(DEV))
+        out = st.step(q.to(DEV), keys_all[:, n0].to(DEV), vals_all[:, n0].to(DEV)).float().cpu().numpy()
+        n = n0 + 1
+        got_codes = st.codes[:, :n].cpu().numpy()
+        score = orc.hamming_score_u32(orc.pack_sign_u32(pre_q)[:, None], codes_o, "blocked")
+        want_idx = orc.topk_stable(score, k)
+        want = orc.sparse_attention(q.numpy(), keys_all.numpy(), vals_all.numpy(), want_idx)
+        if inside == 0:
+            np.testing.assert_array_equal(got_codes, codes_o)
+            np.testing.assert_array_equal(st.idx.cpu().numpy(), want_idx)
+            assert np.abs(out - want).max() <= 1e-5
+        else:   # pragma: no cover - not reached with these seeds
+            print(f"{inside} pre-activations within {margin} of zero: comparing on the GPU's codes")
+            _check_step(kernel, st, q, keys_all[:, n0], vals_all[:, n0], torch.from_numpy(out), n0, dtype)
+    assert inside == 0, "pick another seed: the strict comparison did not run"

@@ -346,6 +346,33 @@ def test_hash_mlp_two_layers(K, B, H, d_hid, dtype):
         assert diff <= 0.005 * pre.size
 
 
+@pytest.mark.parametrize("B,H", [(1, 32), (4, 8)])
+def test_hash_mlp_shipped_flavour_bf16_residue_and_biases(K, B, H):
+    """The hash function the reference ships (config/llama3-8b-spotlight-generation.json: mlp_dims
+    [128,128,128], two layers; mlp_residue defaults to True, spotlight_generation.py:307) in the model's
+    dtype, bf16, with non-zero biases as a trained checkpoint has them: the kernel rounds to bf16 after
+    the matmul, the bias add, SiLU and the residual add of BOTH layers (spotlight_generation.py:229-255).
+    Against the fp64 oracle a bit may differ only where the pre-activation is within 2e-2 of zero;
+    against the reference's own bf16 torch expression at most 0.5 % of the bits differ."""
+    g = _gen(700 + B + H)
+    dtype = torch.bfloat16
+    x = torch.randn(B, H, 128, generator=g).to(dtype)
+    (w1, b1), (w2, b2) = _hash_weights(g, H, [128, 128, 128], dtype, 0.08)
+    got = K.hash_mlp_pack(x.to(DEV), w1.to(DEV), b1.to(DEV), w2.to(DEV), b2.to(DEV), residue=True).cpu().numpy()
+    pre = orc.mlp_hash(x.float().numpy(), [(w1.float().numpy(), b1.float().numpy()),
+                                           (w2.float().numpy(), b2.float().numpy())], residue=True)
+    flips = _flip_report(got, pre, 2e-2)
+    assert flips <= 0.02 * pre.size
+    ref = orc.mlp_hash_torch(x.unsqueeze(2), [(w1[None], b1[None, :, None]), (w2[None], b2[None, :, None])],
+                             residue=True).squeeze(2)
+    want = orc.pack_sign_u32(ref.float().numpy())
+    diff = np.unpackbits(np.bitwise_xor(got, want).view(np.uint8)).sum()
+    assert diff <= 0.005 * pre.size, (int(diff), pre.size)
+    # the many-rows kernel (prompt keys) gives the same bits as the decode-step kernel
+    rows = K.hash_rows_pack(x[:, None].to(DEV), w1.to(DEV), b1.to(DEV), w2.to(DEV), b2.to(DEV), True).cpu().numpy()
+    np.testing.assert_array_equal(rows[:, 0], got)
+
+
 def test_hash_mlp_residue_and_no_bias(K):
     g = _gen(31)
     x = torch.randn(2, 8, 128, generator=g)

@@ -282,3 +282,56 @@ def test_chunked_prefill_equals_one_shot_prefill(mods):
         whole = m(input_ids=nxt, kv_cache=whole.past_key_values)
         part = m(input_ids=nxt, kv_cache=part.past_key_values)
         assert (whole.logits - part.logits).abs().max() < 2e-3
+
+
+@pytest.mark.parametrize("B,gqa", [(1, False), (3, True)])
+@torch.no_grad()
+def test_generate_replaying_its_captured_token_equals_eager_generate(mods, B, gqa):
+    """generate() decodes its first token eagerly and replays one captured HIP graph for the rest
+    (positions, lengths and the budget are read from the device).  With the graph switched off
+    (draft_kwargs["hip_graph"] = False) every token runs eagerly: both must emit the same tokens, over
+    a stretch in which the budget changes several times, for batch 1 and for a batch with the
+    per-kv-head key hash."""
+    conf = copy.deepcopy(CONF)
+    conf["draft_kwargs"].update(max_cache_len=0, gqa_key_hash=gqa)
+    eager_conf = copy.deepcopy(conf)
+    eager_conf["draft_kwargs"]["hip_graph"] = False
+    base = TinyLM(4, 2, 3, seed=11)
+    base2 = copy.deepcopy(base)
+    m = _wrap(mods, "spotlight-generation", base, conf, seed=12)
+    e = _wrap(mods, "spotlight-generation", base2, eager_conf, seed=12)
+    ids = torch.randint(0, 97, (B, 150), generator=torch.Generator().manual_seed(13))
+    got = m.generate(ids, max_new_tokens=40, eos_token_id=[-1])
+    want = e.generate(ids, max_new_tokens=40, eos_token_id=[-1])
+    assert got.shape == (B, 190) and torch.equal(got, want)
+    assert m.timing["graph_tokens"] == 39 and e.timing["graph_tokens"] == 0
+    assert {orc.num_remain(n, 0.9, 8) for n in range(151, 191)} >= {16, 17, 18, 19}   # the budget moved under the graph
+
+
+@torch.no_grad()
+def test_generate_recovers_when_a_bounded_wait_runs_out(mods):
+    """A prompt long enough for two blocks of rows per head, so that the one-launch step exchanges
+    histograms; every such exchange is made to fail from the host (a peer that does not exist, a short
+    poll limit).  generate() sees the error word at its per-token read of the device, moves every layer
+    to token-major codes, takes the token back and decodes it again: the output must equal an
+    undisturbed run's."""
+    from spotlight_amd import _lib
+    L = _lib.load()
+    conf = copy.deepcopy(CONF)
+    conf["draft_kwargs"].update(max_cache_len=0)
+    base = TinyLM(4, 2, 3, seed=21)
+    base2 = copy.deepcopy(base)
+    m = _wrap(mods, "spotlight-generation", base, conf, seed=22)
+    m2 = _wrap(mods, "spotlight-generation", base2, conf, seed=22)
+    ids = torch.randint(0, 97, (1, 700), generator=torch.Generator().manual_seed(23))
+    want = m.generate(ids, max_new_tokens=6, eos_token_id=[-1])
+    _lib.check(L.sl_tune(b"fused_spin_limit", 64), "sl_tune")
+    _lib.check(L.sl_tune(b"fused_phantom_peer", 1), "sl_tune")
+    try:
+        got = m2.generate(ids, max_new_tokens=6, eos_token_id=[-1])
+    finally:
+        _lib.check(L.sl_tune(b"fused_spin_limit", 0), "sl_tune")
+        _lib.check(L.sl_tune(b"fused_phantom_peer", 0), "sl_tune")
+    assert torch.equal(got, want)
+    # one failure (the first decoded token), one recovery; the graph captured afterwards runs on token-major codes
+    assert m2.timing["recoveries"] == 1 and m.timing["recoveries"] == 0
