@@ -53,6 +53,9 @@ def main():
                     help="also run a plain 256 MiB device copy (reference point for HBM byte counters)")
     ap.add_argument("--host-store", action="store_true",
                     help="keep the full K/V store in pinned host memory behind the LRU table (configs with LRU slots)")
+    ap.add_argument("--reuse", type=float, default=None, metavar="P",
+                    help="each token's queries repeat the previous token's with probability P (fresh new keys and values "
+                         "every token): the access pattern an LRU resident table is for; reports its hit rate")
     ap.add_argument("--floor-only", action="store_true",
                     help="only measure what the step's launches cost by themselves (near-empty kernels on the step's grids)")
     ap.add_argument("--codes-layout", default="auto", choices=["auto", "token", "head"],
@@ -115,9 +118,15 @@ def main():
     gpu_gen.manual_seed(0)
 
     # per-token inputs for every layer, drawn once; a token's slice is copied in by the graph
-    P = 16
+    P = 16 if args.reuse is None else 64
     pool = [torch.randn((P, L, B, h, d), generator=gpu_gen, device=dev, dtype=torch.float32).to(dtype)
             for h in (QH, KH, KH)]
+    if args.reuse is not None:
+        # a token keeps the previous token's queries with probability --reuse (decided per token, seeded)
+        coin = torch.rand(P, generator=torch.Generator().manual_seed(3))
+        for i in range(1, P):
+            if coin[i].item() < args.reuse:
+                pool[0][i].copy_(pool[0][i - 1])
     cur = [torch.empty((1, L, B, h, d), device=dev, dtype=dtype) for h in (QH, KH, KH)]
     tok = torch.zeros((1,), dtype=torch.int64, device=dev)
 
@@ -152,6 +161,7 @@ def main():
     for _ in range(tokens_warm - 1):
         token_graph.replay()
     torch.cuda.synchronize()
+    lru_before = [st.lru_stats.sum(dim=(0, 1)).cpu() for st in layers] if c["lru"] else None
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(tokens_timed + 1)]
     t0 = time.perf_counter()
     marks[0].record()
@@ -164,6 +174,13 @@ def main():
     per_token_us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 / L for i in range(tokens_timed))
     ms_per_step = wall_ms / steps_timed
     us_per_step = ms_per_step * 1e3
+    lru_hit_rate = link_gbps = None
+    if c["lru"]:
+        delta = sum((st.lru_stats.sum(dim=(0, 1)).cpu() - b0).to(torch.int64) for st, b0 in zip(layers, lru_before))
+        hits, misses = int(delta[0]), int(delta[1])
+        lru_hit_rate = hits / max(1, hits + misses)
+        # every miss moves one K and one V row from the full store into the resident table
+        link_gbps = misses * 2 * d * (4 if c["dtype"] == "f32" else 2) / (wall_ms * 1e-3) / 1e9
     # a bounded wait that ran out would have produced wrong rows silently: no figure is reported then
     failed = [i for i, st in enumerate(layers) if st.peer_wait_failed()]
     if failed:
@@ -274,6 +291,9 @@ def main():
         "us_per_step_median_token": round(per_token_us[len(per_token_us) // 2], 3),
         "us_per_step_min_token": round(per_token_us[0], 3), "us_per_step_max_token": round(per_token_us[-1], 3),
         "cold_first_token_us": round(cold_first_token_us, 3),
+        "lru_hit_rate": round(lru_hit_rate, 4) if lru_hit_rate is not None else None,
+        "lru_miss_row_gbps": round(link_gbps, 1) if link_gbps is not None else None,
+        "query_reuse": args.reuse,
         "hbm_gbps": round(step_gbps, 1), "hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(ab["step"]),
         "tokens_per_s": round(B / (ms_per_step * 1e-3 * L), 2), "tokens_per_s_layers": L,

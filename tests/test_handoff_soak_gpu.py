@@ -58,7 +58,7 @@ def _pair(env, B, QH, KH, n0, k, lru, seed):
 
 
 @pytest.mark.parametrize("name,B,QH,KH,n0,k,lru", [
-    ("headline shape: fused select + attend, 9 runs per head", 1, 32, 8, 32768, 655, 0),
+    ("headline shape: one-launch scorer + tail, 13 blocks of 2560 rows (= attention runs) per head", 1, 32, 8, 32768, 655, 0),
     ("batch 16 with the LRU table: attention launch with deferred fetch, 2 runs per head", 16, 32, 8, 16384, 328, 1024),
 ])
 @torch.no_grad()
@@ -73,3 +73,4 @@ def test_every_replay_matches_the_run_without_a_hand_off(env, name, B, QH, KH, n
         err = float((a.float() - b.float()).abs().max())
         assert same_idx and err <= 2e-2, f"replay {i}: idx equal {same_idx}, max-abs output difference {err}"
     assert multi.seq_lens.tolist() == single.seq_lens.tolist() == [n0 + REPLAYS] * B
+    assert not multi.peer_wait_failed() and not single.peer_wait_failed()   # no bounded wait ran out in any replay
