@@ -287,14 +287,15 @@ typedef struct {
     /* caches, token-major; codes_head_major != 0: codes are [B, KH, n_cap, W]  */
     /* and scorer, selection and (without an LRU table) attention run as ONE    */
     /* launch; needs W == 4, QH/KH in {1,2,4,5}, n_max <= 262144 (131072 with   */
-    /* an LRU table) and a grid that                                            */
-    /* fits the device at once (sl_decode_head_major_fits): otherwise           */
-    /* SL_ERR_UNSUPPORTED, use token-major codes.  The blocks of that launch    */
-    /* wait for each other (bounded; see sl_decode_error_offset), which assumes */
-    /* the launch gets the whole device: with other kernels running at the same */
-    /* time on other streams prefer token-major codes                           */
+    /* an LRU table) and a head whose blocks of rows fit one XCD's share of the */
+    /* device (sl_decode_head_major_fits): otherwise SL_ERR_UNSUPPORTED, use    */
+    /* token-major codes.  The blocks of a head wait for each other (bounded;   */
+    /* see sl_decode_error_offset), which assumes that workgroups start in the  */
+    /* order of their numbers and that the launch gets the device: with other   */
+    /* kernels running at the same time on other streams prefer token-major     */
+    /* codes                                                                    */
     int codes_head_major;
-    uint32_t *codes;        /* [B, n_cap, KH, W]                                */
+    uint32_t *codes;        /* [B, n_cap, KH, W], or [B, KH, n_cap, W] head-major   */
     void *keys, *vals;      /* [B, n_cap, KH, d]                                */
     int32_t *seq_lens;      /* [B] tokens cached BEFORE this step; incremented  */
     /* outputs */
@@ -334,11 +335,13 @@ size_t sl_decode_workspace_bytes(const sl_decode_params *p);
 size_t sl_decode_error_offset(const sl_decode_params *p);
 /* Whether sl_decode_step can run this shape over head-major codes on the current
  * device: the rows per block it would use (> 0), 0 if it cannot (the caller then
- * keeps token-major codes), negative on bad arguments.  The blocks of rows of such a
- * launch (512 to 8192 rows: the smallest that give a (b, kv head) at most 16 blocks)
- * wait for each other, so B * KH * blocks may not exceed the workgroups the device
- * holds at once; n_max is the largest row bound the caller will pass (its n_cap).
- * No counterpart in the reference. */
+ * keeps token-major codes), negative on bad arguments.  The blocks of rows of a
+ * (b, kv head) in such a launch (512 to 8192 rows: the smallest that give a head at
+ * most 16 blocks -- 32 beyond 64k rows -- and keep the grid on the device at once;
+ * for grids the device cannot hold at once, which then run in rounds, the fewest
+ * blocks per head) wait for each other, so the blocks of ONE head must fit an XCD's
+ * share of the workgroups the device holds; n_max is the largest row bound the
+ * caller will pass (its n_cap).  No counterpart in the reference. */
 int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int k, int with_lru);
 int sl_decode_step(const sl_decode_params *p, void *stream);
 

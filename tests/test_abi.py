@@ -101,3 +101,11 @@ def test_host_budget_formula():
     # spotlight_generation.py:162-164
     for n, mask_out, k in [(4096, 0.9, 410), (16384, 0.98, 328), (32768, 0.98, 656), (131072, 0.98, 2622), (7, 0.98, 7)]:
         assert K.num_remain(n, mask_out) == k
+
+
+def test_product_library_carries_no_phase_stamps(lib):
+    """sl_phase_stamps only answers in the measurement build (-DSL_PHASE_STAMPS); the product library says
+    SL_ERR_UNSUPPORTED without touching its arguments' memory or a GPU."""
+    buf = (C.c_ulonglong * 4)()
+    assert lib.sl_phase_stamps(b"fused", buf, 4, 0) == -3
+    assert lib.sl_phase_stamps(None, None, 0, 0) == -3
