@@ -462,13 +462,13 @@ def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False):
         blocks = (n_max + rows - 1) // rows if rows > 0 else blocks4k
         grids = [grids[0], (blocks * KH * B, 512)]
         if c["lru"]:
-            grids += [(B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
+            grids += [(B * KH, 1024), (min(32, max(1, -(-512 // (B * KH)))) * B * KH, 256)]
     elif c["lru"]:
-        grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
+        grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (B * KH, 1024), (min(32, max(1, -(-512 // (B * KH)))) * B * KH, 256)]
     elif QH // KH in (1, 2, 4) and n_max <= 65536 and c["k"] <= 128 * blocks4k:
         grids += [(blocks4k * KH * B, 512)]
     else:
-        grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (min(16, max(1, 256 // (B * KH))) * B * KH, 256)]
+        grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (min(32, max(1, -(-512 // (B * KH)))) * B * KH, 256)]
     table = torch.zeros(1024, dtype=torch.int32, device=dev)
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     res = {"launches_per_step": len(grids), "grids": grids}

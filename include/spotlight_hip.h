@@ -48,7 +48,7 @@ int sl_version(void);
  * the re-entrancy contract above (host memory, not thread safe; change them
  * only while no other thread is inside the library).  The defaults are what
  * every documented figure was measured with.  Keys:
- * "attn_target_wgs": workgroups the attention launch aims for (default 256);
+ * "attn_target_wgs": workgroups the attention launch aims for (default 512);
  * it decides into how many runs the selected rows of a (b, kv head) are cut;
  * "fuse_select_attend": 1 (default) lets the decode step run selection and
  * attention as one launch when the shapes allow and every 4096-token block keeps

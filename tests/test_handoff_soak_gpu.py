@@ -53,13 +53,13 @@ def _pair(env, B, QH, KH, n0, k, lru, seed):
         single.capture(REPLAYS + 8)
     finally:
         _lib.check(L.sl_tune(b"fuse_select_attend", 1), "sl_tune")
-        _lib.check(L.sl_tune(b"attn_target_wgs", 256), "sl_tune")
+        _lib.check(L.sl_tune(b"attn_target_wgs", 512), "sl_tune")
     return multi, single, inputs, g
 
 
 @pytest.mark.parametrize("name,B,QH,KH,n0,k,lru", [
     ("headline shape: one-launch scorer + tail, 13 blocks of 2560 rows (= attention runs) per head", 1, 32, 8, 32768, 655, 0),
-    ("batch 16 with the LRU table: attention launch with deferred fetch, 2 runs per head", 16, 32, 8, 16384, 328, 1024),
+    ("batch 16 with the LRU table: attention launch with deferred fetch, 4 runs per head", 16, 32, 8, 16384, 328, 1024),
 ])
 @torch.no_grad()
 def test_every_replay_matches_the_run_without_a_hand_off(env, name, B, QH, KH, n0, k, lru):
