@@ -65,18 +65,22 @@ constexpr int LRU_CP = 4;  // 16-byte chunks of K and of V a lane keeps in fligh
 
 // One workgroup per (b, kv head).  Wanted tokens are classified against the
 // token -> slot map; the M victims are the M smallest (stamp, slot) among the
-// slots that were not hit, found with a 4 x 8-bit radix select on the stamp and
-// a stable compaction in slot order (ties at the threshold stamp go to the
-// lowest slot), then paired with the misses in token order.
+// slots that were not hit: a histogram of the ages (step - stamp, clipped) gives the
+// threshold stamp in one pass while the threshold age is below the clip (a 4 x 8-bit
+// radix select on the stamp otherwise), a stable compaction in slot order lists them
+// (ties at the threshold stamp go to the lowest slot), and they are paired with the
+// misses in token order.
+constexpr int LRU_AGE_BINS = 1024;
+
 __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
     __shared__ uint8_t s_flag[LRU_MAX_SLOTS];
     __shared__ int32_t s_miss_tok[LRU_MAX_SLOTS];
     __shared__ int32_t s_miss_item[LRU_MAX_SLOTS];
     __shared__ int32_t s_victim[LRU_MAX_SLOTS];
-    __shared__ uint32_t s_hist[256];
+    __shared__ uint32_t s_hist[LRU_AGE_BINS];
     __shared__ uint32_t s_wave[LRU_THREADS / 64 + 1];
     __shared__ uint32_t s_digit, s_remaining;
-    __shared__ int s_new_in, s_new_pos;
+    __shared__ int s_new_in, s_new_pos, s_age[2];
 
     SL_TS(0);   // start
     const int tid = threadIdx.x;
@@ -92,8 +96,18 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
     const uint32_t t = a.stamp + (a.stamp_dev ? a.stamp_dev[0] : 0u);
     const int new_tok = a.new_token ? a.new_token[b] : -1;
 
+    // the stamps of the lane's slots are requested now and used after the classification (a slot that
+    // is hit gets a new stamp below, but a hit slot is no candidate, so the old value is never looked at)
+    const int SPT = (C + LRU_THREADS - 1) / LRU_THREADS;
+    uint32_t key[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int s = tid * SPT + j;
+        key[j] = ss[(j < SPT && s < C) ? s : 0];
+    }
     for (int s = tid; s < C; s += LRU_THREADS) s_flag[s] = 0;
-    if (tid == 0) { s_new_in = 0; s_new_pos = -1; }
+    if (tid == 0) { s_new_in = 0; s_new_pos = -1; s_age[0] = -1; s_age[1] = 0; }
+    if (tid < LRU_AGE_BINS) s_hist[tid] = 0;
     __syncthreads();
 
     // wanted items 0..k-1 = idx, item k = the new token unless idx already holds it
@@ -150,16 +164,37 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
 
     SL_TS(1);   // wanted rows classified against the map, misses listed
     if (M > 0) {
-        const int SPT = (C + LRU_THREADS - 1) / LRU_THREADS;
-        uint32_t key[4];
+        // slots that were not hit (empty ones included, stamp 0) are the candidates; their stamps are the ones loaded above
         bool elig[4];
+        uint32_t age[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int s = tid * SPT + j;
             elig[j] = j < SPT && s < C && s_flag[s] == 0;
-            key[j] = elig[j] ? ss[s] : 0u;
+            if (!elig[j]) key[j] = 0u;
+            age[j] = t - key[j];
+            age[j] = age[j] < LRU_AGE_BINS - 1 ? age[j] : LRU_AGE_BINS - 1;
+            if (elig[j]) atomicAdd(&s_hist[age[j]], 1u);
         }
-        // stamps are step numbers: the high bytes are usually all zero, and a radix
+        __syncthreads();
+        // the M oldest: walk the ages from the largest; lane tid owns age LRU_AGE_BINS-1-tid
+        {
+            const uint32_t c = s_hist[LRU_AGE_BINS - 1 - tid];
+            uint32_t all;
+            const uint32_t before = block_exclusive_sum<LRU_THREADS>(c, s_wave, &all);
+            if (before < static_cast<uint32_t>(M) && before + c >= static_cast<uint32_t>(M)) {
+                s_age[0] = LRU_AGE_BINS - 1 - tid;
+                s_age[1] = static_cast<int>(static_cast<uint32_t>(M) - before);
+            }
+        }
+        __syncthreads();
+        uint32_t prefix, remaining;
+        if (s_age[0] >= 0 && s_age[0] < LRU_AGE_BINS - 1) {
+            prefix = t - static_cast<uint32_t>(s_age[0]);
+            remaining = static_cast<uint32_t>(s_age[1]);
+        } else {
+        // the threshold lies among the ages the histogram clips together: select on the stamp itself.
+        // Stamps are step numbers: the high bytes are usually all zero, and a radix
         // pass over a byte that is zero in every key selects nothing -- skip those
         uint32_t kmax = 0;
 #pragma unroll
@@ -176,7 +211,8 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
         const uint32_t all_max = s_digit;
         const int first_pass = all_max < (1u << 8) ? 3 : all_max < (1u << 16) ? 2 : all_max < (1u << 24) ? 1 : 0;
         __syncthreads();  // s_digit is rewritten by the passes
-        uint32_t prefix = 0, remaining = static_cast<uint32_t>(M);
+        prefix = 0;
+        remaining = static_cast<uint32_t>(M);
         for (int pass = first_pass; pass < 4; ++pass) {
             const int shift = 24 - 8 * pass;
             const uint32_t hi_mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
@@ -204,7 +240,8 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(lru_args a) {
             prefix |= s_digit << shift;
             remaining = s_remaining;
         }
-        SL_TS(2);   // radix passes done: threshold stamp known
+        }
+        SL_TS(2);   // threshold stamp known
         const uint32_t thr = prefix, need_eq = remaining;
         uint32_t lt = 0, eq = 0;
 #pragma unroll

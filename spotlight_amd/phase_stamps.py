@@ -26,7 +26,7 @@ POINTS = {
               10: "attention: query slices requested", 11: "chunk 0: K / V loads issued", 12: "chunk 0: scores done (K rows arrived)",
               13: "chunk 0: probabilities in LDS", 14: "all chunks accumulated", 15: "wave tiles in LDS", 16: "partials stored",
               17: "partials acknowledged", 18: "ticket taken", 19: "merge: loads of all runs issued", 20: "merged output stored"},
-    "lru": {0: "start", 1: "wanted rows classified, misses listed", 2: "radix passes done", 3: "victims listed", 4: "table updated"},
+    "lru": {0: "start", 1: "wanted rows classified, misses listed", 2: "threshold stamp known", 3: "victims listed", 4: "table updated"},
 }
 POINTS["attn"] = {k: v for k, v in POINTS["fused"].items() if k >= 10}
 POINTS["select_attend"] = POINTS["attn"]

@@ -191,8 +191,11 @@ def _lru_call(kernel, lib, L, idx, new_tok, st, ss, ts, keys, vals, kres, vres, 
     return slots, stats
 
 
+# `scale` spreads the stamps: with 1 every age stays small (the victims' threshold comes from the age
+# histogram), with 700 the oldest slots are older than the histogram resolves (the select on the stamp runs)
+@pytest.mark.parametrize("scale", [1, 700])
 @pytest.mark.parametrize("C,k,n0,steps", [(8, 3, 12, 40), (64, 20, 100, 30), (1024, 328, 2000, 6), (4096, 1000, 5000, 3)])
-def test_lru_matches_bruteforce_model(env, C, k, n0, steps):
+def test_lru_matches_bruteforce_model(env, C, k, n0, steps, scale):
     decode, kernel = env
     from spotlight_amd import _lib as lib
     L = lib.load()
@@ -208,13 +211,14 @@ def test_lru_matches_bruteforce_model(env, C, k, n0, steps):
     vres = torch.zeros_like(kres)
     models = [[orc.LruModel(C) for _ in range(KH)] for _ in range(B)]
     n = n0
-    for t in range(1, steps + 1):
+    for step in range(1, steps + 1):
+        t = step * scale
         idx = np.zeros((B, KH, k), dtype=np.int32)
         for b in range(B):
             for h in range(KH):
                 sel = r.choice(n, size=k, replace=False)
                 res = [x for x in models[b][h].token if x >= 0]
-                if res and t % 2 == 0:      # re-use resident tokens so that hits occur
+                if res and step % 2 == 0:      # re-use resident tokens so that hits occur
                     take = min(len(res), k // 2)
                     sel = np.unique(np.concatenate([r.choice(res, size=take, replace=False), sel]))[:k]
                     while len(sel) < k:
