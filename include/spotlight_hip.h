@@ -339,7 +339,9 @@ size_t sl_decode_error_offset(const sl_decode_params *p);
  * (b, kv head) in such a launch (512 to 8192 rows: the smallest that give a head at
  * most 16 blocks -- 32 beyond 64k rows -- and keep the grid on the device at once;
  * for grids the device cannot hold at once, which then run in rounds, the fewest
- * blocks per head) wait for each other, so the blocks of ONE head must fit an XCD's
+ * blocks per head that make the grid at least 1.75 times what the device holds;
+ * with an LRU table blocks of 4096 rows, 3072 or 8192 where those suit the shape)
+ * wait for each other, so the blocks of ONE head must fit an XCD's
  * share of the workgroups the device holds; n_max is the largest row bound the
  * caller will pass (its n_cap).  No counterpart in the reference. */
 int sl_decode_head_major_fits(int dtype, int B, int QH, int KH, int nbits, int64_t n_max, int k, int with_lru);

@@ -354,9 +354,10 @@ int slots_rows(int slots_per_lane, bool many) {
 // blocks measured slower again, and so did more than 8 rows per lane, which therefore only come in where
 // fewer, larger blocks are what it takes to keep the grid resident: batch 8 at 32k rows; 128k rows: 29
 // blocks of 4608 rows 24.6 us against 30.2 with 17 of 8192).  A grid the device cannot hold at once
-// (large batches) runs in rounds: then the fewest blocks per head, and the smallest rows per block that
-// give that few.  Without the attention (LRU table): 4096 rows where that fits (3072 in the case
-// described below), else 8192.
+// (large batches) runs in rounds: then the fewest blocks per head that still make the grid 1.75 times what
+// the device holds, and the smallest rows per block that give that few.  Without the attention (LRU
+// table): 4096 rows, in rounds where the grid is large (3072 in the case described below), 8192 only
+// for caches too long for those.
 template <typename T, int G, bool ATTEND>
 int pick_rows(int64_t n, int64_t heads, int peer_cap) {
     if (n < 1) n = 1;
@@ -379,15 +380,23 @@ int pick_rows(int64_t n, int64_t heads, int peer_cap) {
         if (ATTEND) return (heads + SL_XCDS - 1) / SL_XCDS * blocks_of(spl) <= slots / SL_XCDS;
         return heads * blocks_of(spl) <= slots;
     };
-    // a grid that runs in rounds: fewest blocks per head, then the smallest rows per block with that few
+    // a grid that runs in rounds: the fewest blocks per head (then the smallest rows per block with that
+    // few) that still make the grid at least 1.75 times what the device holds at once -- a grid just over
+    // one round leaves most of the device idle in its last round, and workgroups of different rounds fill
+    // each other's waiting phases (32k rows, batch 16: 7 blocks of 5120 rows 57.5 us against 5 of 7168
+    // 62.4; from batch 32 on 5 blocks of 7168 rows already give 2.5 rounds and measured fastest)
     auto in_rounds = [&](const int *flavours, int count) {
-        int best = 0;
+        int best = 0, most = 0;
         for (int i = 0; i < count; ++i) {
             const int f = flavours[i];
             if (!runs(f)) continue;
+            if (most == 0 || blocks_of(f) > blocks_of(most)) most = f;
+            const int slots = slots_rows<T, G, ATTEND>(f, blocks_of(f) > 16);
+            const int64_t grid = ATTEND ? (heads + SL_XCDS - 1) / SL_XCDS * blocks_of(f) * SL_XCDS : heads * blocks_of(f);
+            if (4 * grid < 7 * static_cast<int64_t>(slots)) continue;
             if (best == 0 || blocks_of(f) < blocks_of(best)) best = f;
         }
-        return best;
+        return best ? best : most;
     };
     int spl = 0;
     if (g_fused_rows) spl = g_fused_rows % 512 == 0 && runs(g_fused_rows / 512) ? g_fused_rows / 512 : 0;
@@ -403,17 +412,19 @@ int pick_rows(int64_t n, int64_t heads, int peer_cap) {
                 if (fits(f) && heads * blocks_of(f) <= cus) { spl = f; break; }
         if (spl == 0) spl = in_rounds(FS_FLAVOURS, static_cast<int>(sizeof(FS_FLAVOURS) / sizeof(FS_FLAVOURS[0])));
     } else {
-        // many workgroups per compute unit here (large batches): blocks of 3072 rows where they need
-        // no more rounds of workgroups over the device than blocks of 4096 (C3: 768 workgroups, three
-        // per compute unit, 15.6 us against 17.3 with 640 of 4096 rows)
-        spl = fits(8) ? 8 : fits(16) ? 16 : 0;
-        if (spl == 8 && fits(6)) {
+        // many workgroups per compute unit here (large batches): blocks of 4096 rows, in as many rounds
+        // as the grid takes (batch 32 x 16k rows: 1280 workgroups of 4096 rows 27.4 us, 1536 of 3072
+        // rows 28.2, 768 of 8192 rows -- which the device holds at once -- 51.2; batch 64: 46.1 / 48.6 /
+        // 88.9), and blocks of 3072 rows where the grid is on the device at once and they need no more
+        // rounds of workgroups over the compute units than blocks of 4096 (C3: 768 workgroups, three per
+        // compute unit, 15.6 us against 17.3 with 640 of 4096 rows).  8192 rows only for caches too long
+        // for the smaller blocks.
+        spl = runs(8) ? 8 : runs(16) ? 16 : 0;
+        if (spl == 8 && fits(8) && fits(6)) {
             const int64_t cus = sl_compute_units();
             const int64_t w6 = heads * ((n + 3071) / 3072), w8 = heads * ((n + 4095) / 4096);
             if (cus > 0 && (w6 + cus - 1) / cus <= (w8 + cus - 1) / cus) spl = 6;
         }
-        static const int lru_flavours[] = {6, 8, 16};
-        if (spl == 0) spl = in_rounds(lru_flavours, 3);
     }
     return spl == 0 && unknown ? -1 : 512 * spl;
 }

@@ -737,7 +737,8 @@ def test_head_major_grids_larger_than_the_device_run_in_rounds(env):
     try:
         for case, (B, KH, G, n0, k, rows, lru) in enumerate([(64, 8, 4, 1500, 30, 512, 0), (48, 8, 1, 3000, 64, 1024, 0),
                                                              (32, 8, 4, 2500, 50, 0, 0), (64, 4, 2, 5000, 100, 1024, 0),
-                                                             (64, 8, 4, 7000, 60, 3072, 128), (40, 8, 5, 2000, 40, 512, 0)]):
+                                                             (64, 8, 4, 7000, 60, 3072, 128), (40, 8, 5, 2000, 40, 512, 0),
+                                                             (64, 8, 4, 9000, 60, 0, 128), (24, 8, 4, 24000, 100, 0, 0)]):
             QH = KH * G
             n_cap = (n0 + 16 + 7) // 8 * 8
             cg = torch.Generator().manual_seed(900 + case)
