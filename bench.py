@@ -111,7 +111,8 @@ def main():
         blocks = (n_cap + 4095) // 4096
         head = args.codes_layout == "head" or (args.codes_layout == "auto" and not c["lru"] and QH // KH in (1, 2, 4)
                                                and n_cap <= 65536 and B * KH * blocks <= 256 and k <= 128 * blocks)
-        print(json.dumps({"config": args.config, "latency_floor": latency_floor(dev, c, L, n0 + tokens, reps=64, one_launch_tail=head)}), flush=True)
+        print(json.dumps({"config": args.config, "latency_floor": latency_floor(dev, c, L, n0 + tokens, reps=64, one_launch_tail=head,
+                                                                                   lru_inside=lru_inside_selection_launch(c, args.tune, head))}), flush=True)
         return
 
     gpu_gen = torch.Generator(device=dev)
@@ -263,7 +264,8 @@ def main():
                     "algorithmic_bytes_per_launch": kernels[dominant]["algorithmic_bytes"],
                     "us_per_launch": kernels[dominant]["us"]}
 
-    floor = latency_floor(dev, c, L, n_max, one_launch_tail=layers[0].codes_layout == "head")
+    lru_inside = lru_inside_selection_launch(c, args.tune, layers[0].codes_layout == "head")
+    floor = latency_floor(dev, c, L, n_max, one_launch_tail=layers[0].codes_layout == "head", lru_inside=lru_inside)
 
     cpu_baseline = cpu_reference_form = None
     if not args.no_cpu_baseline:
@@ -297,7 +299,7 @@ def main():
         "hbm_gbps": round(step_gbps, 1), "hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(ab["step"]),
         "tokens_per_s": round(B / (ms_per_step * 1e-3 * L), 2), "tokens_per_s_layers": L,
-        "kernels": kernels, "roofline": roofline, "cpu_baseline": cpu_baseline,
+        "kernels": kernels, "lru_inside_selection_launch": lru_inside, "roofline": roofline, "cpu_baseline": cpu_baseline,
         "cpu_baseline_reference_form": cpu_reference_form,
         "latency_floor": floor,
         "value_over_floor": round(us_per_step / floor["launches_with_one_load_us"], 2) if floor else None,
@@ -440,7 +442,13 @@ def profiled_traffic(config, stage):
     return None
 
 
-def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False):
+def lru_inside_selection_launch(c, tunes, one_launch_tail):
+    """Whether the step's scorer + selection launch also runs the table update (the library's rule:
+    head-major codes, a table of at most 2048 slots, not switched off with --tune fused_lru=0)."""
+    return bool(one_launch_tail and c["lru"] and c["lru"] <= 2048 and "fused_lru=0" not in tunes)
+
+
+def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False, lru_inside=False):
     """What the step's launches cost by themselves on this machine: a HIP graph of L x (as many dependent
     launches as the step has, with the step's grids) of a kernel that does nothing, and of one whose lanes do a
     single dependent load.  us per step-equivalent."""
@@ -462,7 +470,7 @@ def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False):
         blocks = (n_max + rows - 1) // rows if rows > 0 else blocks4k
         grids = [grids[0], (blocks * KH * B, 512)]
         if c["lru"]:
-            grids += [(B * KH, 1024), (min(32, max(1, -(-512 // (B * KH)))) * B * KH, 256)]
+            grids += ([] if lru_inside else [(B * KH, 1024)]) + [(min(32, max(1, -(-512 // (B * KH)))) * B * KH, 256)]
     elif c["lru"]:
         grids += [(((n_max + 8191) // 8192) * B * KH, 1024), (B * KH, 1024), (min(32, max(1, -(-512 // (B * KH)))) * B * KH, 256)]
     elif QH // KH in (1, 2, 4) and n_max <= 65536 and c["k"] <= 128 * blocks4k:

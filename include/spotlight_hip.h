@@ -67,6 +67,10 @@ int sl_version(void);
  * step -- polls before a workgroup gives up (0 = the default, 2^22) and 1 = every
  * head also waits for a block that does not exist, so that each workgroup gives
  * up after the limit, sets the error word and the launch still drains;
+ * "fused_lru": 1 (default) lets the scorer + selection launch of a whole step over
+ * head-major codes end with the resident-table update (tables of up to 2048 slots:
+ * the block of a (b, kv head) that finishes last runs it), 0 keeps the update a
+ * launch of its own;
  * "hist_copies": copies of the score histogram (4, 8, 16 or 32; 0 = by cache
  * length), to be set before any workspace is sized. */
 int sl_tune(const char *key, int value);

@@ -254,9 +254,26 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
     aa.keys = p.keys; aa.vals = p.vals; aa.idx = p.idx;
     aa.kv_stride_b = p.n_cap * p.KH * p.d; aa.kv_stride_h = p.d;
     aa.kv_stride_n = static_cast<int64_t>(p.KH) * p.d;
+    // resident-table update, where there is a table
+    lru_args la{};
+    bool lru_done = false;
+    const bool defer = (stages & SL_STAGE_LRU) && (stages & SL_STAGE_ATTN);
+    int32_t *fetch = reinterpret_cast<int32_t *>(ws + L.lru_fetch);
+    if (p.lru_C > 0) {
+        SL_REQUIRE(p.k + 1 <= p.lru_C && p.lru_C <= LRU_MAX_SLOTS, SL_ERR_UNSUPPORTED);
+        la.idx = p.idx; la.new_token = p.seq_lens; la.slot_token = p.slot_token; la.slot_stamp = p.slot_stamp;
+        la.token_slot = p.token_slot; la.keys = p.keys; la.vals = p.vals; la.k_res = p.k_res; la.v_res = p.v_res;
+        la.slots_out = p.slots_out; la.stats = p.lru_stats; la.stamp_dev = p.step_counter; la.stamp = 1;
+        la.dtype = p.dtype; la.B = p.B; la.KH = p.KH; la.d = p.d; la.k = p.k; la.C = p.lru_C;
+        la.map_cap = p.lru_map_cap; la.kv_stride_b = p.n_cap * p.KH * p.d;
+        // When the attention follows in the same call, it fetches the rows of the selected
+        // misses from the full store itself (it has to read them anyway) and drops them
+        // into their slots: the table update then copies no rows but the new token's.
+        la.fetch_out = defer ? fetch : nullptr;
+    }
     if (p.codes_head_major) {
-        // hash, then scorer + selection (+ attention, unless an LRU table update comes in between) as ONE
-        // launch over head-major codes
+        // hash, then scorer + selection (+ attention, or -- with an LRU table -- the table update of each
+        // head by the block that finishes last) as ONE launch over head-major codes
         SL_REQUIRE(sl_fused_step_supported(G, W, G * p.nbits + 1, p.n_max, p.B, p.KH), SL_ERR_UNSUPPORTED);
         const bool attend = p.lru_C == 0;
         const int one = SL_STAGE_SCORE | SL_STAGE_SELECT | (attend ? SL_STAGE_ATTN : 0);
@@ -275,6 +292,11 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
             select_args fs{};
             fs.B = p.B; fs.KH = p.KH; fs.n_bins = G * p.nbits + 1; fs.idx = p.idx; fs.seq_lens = n_rows; fs.keep = keep_rows;
             fs.k = p.k; fs.len_bias = 0; fs.n = p.n_max;
+            if (!attend && whole && g_fused_lru && p.lru_C <= FS_LRU_MAX_SLOTS) {
+                fa.lru_on = 1;
+                fa.lru = la;
+                lru_done = true;
+            }
             rc = sl_fused_step_launch(fa, fs, aa, attend, ws + L.fused, ws + L.attn, attn_bytes, s);
             if (rc != SL_OK || attend) return rc;
         }
@@ -326,22 +348,9 @@ extern "C" int sl_decode_stages(const sl_decode_params *pp, int stages, void *st
         }
     }
 
-    // 4. optional LRU, 5. attention
+    // 4. optional LRU (unless the scorer + selection launch has run it), 5. attention
     if (p.lru_C > 0) {
-        SL_REQUIRE(p.k + 1 <= p.lru_C && p.lru_C <= LRU_MAX_SLOTS, SL_ERR_UNSUPPORTED);
-        lru_args la{};
-        la.idx = p.idx; la.new_token = p.seq_lens; la.slot_token = p.slot_token; la.slot_stamp = p.slot_stamp;
-        la.token_slot = p.token_slot; la.keys = p.keys; la.vals = p.vals; la.k_res = p.k_res; la.v_res = p.v_res;
-        la.slots_out = p.slots_out; la.stats = p.lru_stats; la.stamp_dev = p.step_counter; la.stamp = 1;
-        la.dtype = p.dtype; la.B = p.B; la.KH = p.KH; la.d = p.d; la.k = p.k; la.C = p.lru_C;
-        la.map_cap = p.lru_map_cap; la.kv_stride_b = p.n_cap * p.KH * p.d;
-        // When the attention follows in the same call, it fetches the rows of the selected
-        // misses from the full store itself (it has to read them anyway) and drops them
-        // into their slots: the table update then copies no rows but the new token's.
-        const bool defer = (stages & SL_STAGE_LRU) && (stages & SL_STAGE_ATTN);
-        int32_t *fetch = reinterpret_cast<int32_t *>(ws + L.lru_fetch);
-        la.fetch_out = defer ? fetch : nullptr;
-        if (stages & SL_STAGE_LRU) {
+        if ((stages & SL_STAGE_LRU) && !lru_done) {
             rc = sl_lru_launch(la, s);
             if (rc != SL_OK) return rc;
         }

@@ -1,6 +1,7 @@
 // Scorer + count-select + sparse attention as one launch over head-major key codes.
 #pragma once
 #include "attn.h"
+#include "lru.h"
 #include "topk.h"
 
 constexpr int FS_MAX_PEERS = 32;   // most blocks of rows (512 ... 8192) per (b, kv head)
@@ -20,7 +21,11 @@ struct fused_args {
     uint32_t spin_limit;      // polls before giving up (set by the launcher)
     unsigned blocks;          // blocks of rows per (b, kv head) the grid was sized for (set by the launcher)
     int phantom_peers;        // 0; 1 = also wait for a block that does not exist (test of the bounded wait)
+    int lru_on;               // launches without the attention: 1 = the block of a (b, kv head) that finishes last
+    lru_args lru;             // runs the resident-table update `lru` over the head's list (lru.idx = the list,
+                              // lru.fetch_out given, lru.C <= FS_LRU_MAX_SLOTS) before the launch ends
 };
+constexpr int FS_LRU_MAX_SLOTS = 2048;   // largest resident table the launch updates itself (8-wave workgroups, 4 slots per lane)
 
 size_t sl_fused_ws_bytes(int B, int KH, int peer_cap);
 bool sl_fused_step_supported(int G, int W, int n_bins, int64_t n, int B, int KH);
@@ -44,4 +49,5 @@ SL_FUSED_DECL(bf16_g1) SL_FUSED_DECL(bf16_g2) SL_FUSED_DECL(bf16_g4) SL_FUSED_DE
 SL_FUSED_DECL(f16_g1) SL_FUSED_DECL(f16_g2) SL_FUSED_DECL(f16_g4) SL_FUSED_DECL(f16_g5)
 #undef SL_FUSED_DECL
 extern int g_fused_rows;                       // sl_tune("fused_rows")
+extern int g_fused_lru;                        // sl_tune("fused_lru", 0 | 1): table update inside the scorer + selection launch
 constexpr uint32_t FS_SPIN_LIMIT = 1u << 22;   // polls a workgroup waits for a peer before it gives up (fused_args::spin_limit)

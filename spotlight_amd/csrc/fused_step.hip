@@ -30,6 +30,7 @@ int g_fused_rows = 0;  // sl_tune("fused_rows", 0 | multiple of 512): rows per b
 // wait -- a short limit and a peer that does not exist make every workgroup give up and report it
 static uint32_t g_fused_spin_limit = FS_SPIN_LIMIT;
 static int g_fused_phantom_peer = 0;
+int g_fused_lru = 1;   // sl_tune("fused_lru", 0): the table update as a launch of its own after the scorer + selection launch
 
 size_t sl_fused_ws_bytes(int B, int KH, int peer_cap) {
     const size_t bh = static_cast<size_t>(B) * KH;
@@ -47,6 +48,7 @@ int sl_fused_tune(const char *key, int value) {
     }
     if (!strcmp(key, "fused_spin_limit") && value >= 0) { g_fused_spin_limit = value ? static_cast<uint32_t>(value) : FS_SPIN_LIMIT; return SL_OK; }
     if (!strcmp(key, "fused_phantom_peer") && (value == 0 || value == 1)) { g_fused_phantom_peer = value; return SL_OK; }
+    if (!strcmp(key, "fused_lru") && (value == 0 || value == 1)) { g_fused_lru = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
 
@@ -105,6 +107,15 @@ int sl_fused_step_launch(fused_args fa, select_args sa, attn_args aa, bool atten
     aa.peer_flag_stride = fa.peer_cap;
     fa.spin_limit = g_fused_spin_limit;
     fa.phantom_peers = g_fused_phantom_peer;   // (the launcher drops it where a head has no free flag)
+    if (fa.lru_on) {
+        // the table update at the end of the launch: over this launch's own list, rows of the misses left
+        // to the consumer, a table the 8-wave workgroup covers with 4 slots per lane
+        const lru_args &la = fa.lru;
+        SL_REQUIRE(!attend && la.idx == sa.idx && la.k == sa.k && la.B == aa.B && la.KH == aa.KH, SL_ERR_SHAPE);
+        SL_REQUIRE(la.fetch_out && la.slots_out && la.slot_token && la.slot_stamp && la.token_slot && la.keys && la.vals &&
+                   la.k_res && la.v_res && la.new_token, SL_ERR_NULL);
+        SL_REQUIRE(la.k + 1 <= la.C && la.C <= FS_LRU_MAX_SLOTS && la.map_cap > 0, SL_ERR_UNSUPPORTED);
+    }
     switch (aa.dtype) {
         case SL_F32: return launch_f32(G, fa, sa, aa, attend, s);
         case SL_BF16: return launch_bf16(G, fa, sa, aa, attend, s);

@@ -10,6 +10,7 @@
 #endif
 #include "phase_stamps.h"
 #include "attn_core.h"
+#include "lru_core.h"
 #include "topk_core.h"
 
 namespace {
@@ -20,6 +21,17 @@ constexpr int FS_THREADS = FS_NW * 64;
 constexpr int FS_MAX_BPT = 2;                        // histogram bins per lane (<= 1024 bins: sl_fused_step_supported)
 
 static_assert(FS_MAX_PEERS == AT_PART_SPLITS, "one attention run per block of rows");
+
+// The two large LDS tables of the kernel.  A launch without the attention may end with the resident-table
+// update of the head (fused_args::lru_on): its tables take the place of these two once the list is out.
+template <int FS_BLOCK, bool WITH_LRU> union fused_lds;
+template <int FS_BLOCK> union fused_lds<FS_BLOCK, false> {
+    struct { uint32_t hist[FS_THREADS * FS_MAX_BPT]; int32_t list[FS_BLOCK]; } sel;
+};
+template <int FS_BLOCK> union fused_lds<FS_BLOCK, true> {
+    struct { uint32_t hist[FS_THREADS * FS_MAX_BPT]; int32_t list[FS_BLOCK]; } sel;
+    lru_shared<FS_THREADS, FS_LRU_MAX_SLOTS> lru;
+};
 
 // FS_SLOTS rows per lane (row = block start + wave * 64 FS_SLOTS + slot * 64 + lane): blocks of
 // 512 FS_SLOTS rows; pick_rows chooses the size by shape.
@@ -33,10 +45,12 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     constexpr int FS_BLOCK = FS_THREADS * FS_SLOTS;
     __shared__ uint32_t s_wave[64];
     __shared__ int s_tn[4];
-    __shared__ uint32_t s_hist[FS_THREADS * FS_MAX_BPT];
+    __shared__ fused_lds<FS_BLOCK, !ATTEND> s_big;
+    uint32_t (&s_hist)[FS_THREADS * FS_MAX_BPT] = s_big.sel.hist;
+    int32_t (&s_list)[FS_BLOCK] = s_big.sel.list;
     __shared__ uint32_t s_cnt[FS_NW];
     __shared__ int s_range[2];
-    __shared__ int32_t s_list[FS_BLOCK];
+    __shared__ int s_last;
     __shared__ attn_shared<ATTEND ? G : 1, FS_NW> sh;
 
     SL_TS(0);   // start
@@ -76,8 +90,13 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     int k_eff;
     rows_and_keep(sa, b, n_b, k_eff);
     int32_t *out = sa.idx + static_cast<int64_t>(bh) * sa.k;
+    // (without the attention the list may be read in this launch, by the block that runs the table
+    // update: those stores are agent-scope)
     if (blk == 0)
-        for (int i = k_eff + tid; i < sa.k; i += FS_THREADS) out[i] = -1;
+        for (int i = k_eff + tid; i < sa.k; i += FS_THREADS) {
+            if constexpr (ATTEND) out[i] = -1;
+            else st_agent(reinterpret_cast<uint32_t *>(out + i), 0xffffffffu);
+        }
     if (n_b == 0) {
         // no rows at all (a subset of stages run before any hash launch left a row count): nothing is
         // kept, and the attention over nothing is zero
@@ -234,19 +253,47 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
     // the list goes out with coalesced stores; the attention then runs over it
     __syncthreads();
     SL_TS(7);   // kept rows listed in LDS
-    for (int i = tid; i < n_kept; i += FS_THREADS) out[first + i] = s_list[i];
+    for (int i = tid; i < n_kept; i += FS_THREADS) {
+        if constexpr (ATTEND) out[first + i] = s_list[i];
+        else {
+            // (with the table update at the end of the launch every block looks its own rows up in the
+            // token -> slot map, which that update is the only one to change, and leaves the slots
+            // beside the list: the lookups of a head's blocks overlap instead of waiting for the last)
+            const int tok = s_list[i];
+            st_agent(reinterpret_cast<uint32_t *>(out + first + i), static_cast<uint32_t>(tok));
+            if (fa.lru_on) {
+                const int32_t held_in = tok < fa.lru.map_cap ? fa.lru.token_slot[static_cast<int64_t>(bh) * fa.lru.map_cap + tok] : -1;
+                st_agent(reinterpret_cast<uint32_t *>(fa.lru.slots_out + static_cast<int64_t>(bh) * sa.k + first + i), static_cast<uint32_t>(held_in));
+            }
+        }
+    }
     if constexpr (ATTEND) {
         attend_rows_and_merge<T, G, FS_NW, false, false, MAXS>(aa, b, h, blk, S, s_list, n_kept, sh);
     } else {
         // every lane of this block has used what it read from its peers (the barrier above): the last
-        // block of the head to get here lowers the flags for the next launch
-        if (S > 1 && wave == 0) {
-            uint32_t last = 0;
-            if (lane == 0) last = arrive_last(&aa.counter[bh], static_cast<uint32_t>(S)) ? 1u : 0u;
-            if (__builtin_amdgcn_readfirstlane(last)) {
-                if (lane < S) st_agent(fa.peer_flag + static_cast<int64_t>(bh) * fa.peer_cap + lane, 0u);
-                if (lane == 0) st_agent(&aa.counter[bh], 0u);
+        // block of the head to get here lowers the flags for the next launch -- and, with lru_on, runs
+        // the head's table update over the complete list: every block waits until its part of the list
+        // is acknowledged before it takes its ticket
+        const bool epilogue = fa.lru_on != 0;
+        if (epilogue) {
+            publish_wait();
+            __syncthreads();
+        }
+        if (wave == 0) {
+            uint32_t last = S > 1 ? 0u : 1u;
+            if (S > 1) {
+                if (lane == 0) last = arrive_last(&aa.counter[bh], static_cast<uint32_t>(S)) ? 1u : 0u;
+                last = __builtin_amdgcn_readfirstlane(last);
+                if (last) {
+                    if (lane < S) st_agent(fa.peer_flag + static_cast<int64_t>(bh) * fa.peer_cap + lane, 0u);
+                    if (lane == 0) st_agent(&aa.counter[bh], 0u);
+                }
             }
+            if (lane == 0) s_last = static_cast<int>(last);
+        }
+        if (epilogue) {
+            __syncthreads();   // s_last; and nobody reads s_list any more
+            if (s_last) lru_update<FS_THREADS, FS_LRU_MAX_SLOTS, false, true, true, 8>(fa.lru, b, h, s_big.lru, static_cast<int>(n_b) - 1);   // (whole steps only: the head's last row is the new token)
         }
     }
 }

@@ -23,12 +23,14 @@ POINTS = {
     "fused": {0: "start", 1: "row count known, histogram cleared", 2: "codes arrived, scores counted",
               3: "own histogram published and acknowledged", 4: "every peer's flag seen", 5: "peers' bins read and summed",
               6: "threshold known", 7: "kept rows listed in LDS",
+              8: "table update: list acknowledged, ticket won", 9: "table update: wanted rows classified, misses listed",
+              21: "table update: threshold stamp known", 22: "table update: victims listed", 23: "table update: table updated",
               10: "attention: query slices requested", 11: "chunk 0: K / V loads issued", 12: "chunk 0: scores done (K rows arrived)",
               13: "chunk 0: probabilities in LDS", 14: "all chunks accumulated", 15: "wave tiles in LDS", 16: "partials stored",
               17: "partials acknowledged", 18: "ticket taken", 19: "merge: loads of all runs issued", 20: "merged output stored"},
     "lru": {0: "start", 1: "wanted rows classified, misses listed", 2: "threshold stamp known", 3: "victims listed", 4: "table updated"},
 }
-POINTS["attn"] = {k: v for k, v in POINTS["fused"].items() if k >= 10}
+POINTS["attn"] = {k: v for k, v in POINTS["fused"].items() if 10 <= k <= 20}
 POINTS["select_attend"] = POINTS["attn"]
 
 

@@ -298,6 +298,45 @@ def test_decode_with_lru_gives_identical_attention(env, fuse, layout):
         _lib.check(L.sl_tune(b"fuse_select_attend", 1), "sl_tune")
 
 
+@pytest.mark.parametrize("n0,k,C,rows", [(700, 30, 64, 0), (9000, 150, 1024, 3072), (9000, 150, 2048, 0), (20000, 300, 512, 4096),
+                                         (9000, 150, 4096, 0)])
+def test_table_update_inside_the_selection_launch_equals_the_launch_of_its_own(env, n0, k, C, rows):
+    """Over head-major codes the block of a (b, kv head) that finishes last runs the head's table update
+    at the end of the scorer + selection launch (tables of up to 2048 slots; larger ones keep the launch
+    of their own).  Both forms must leave identical tables, slot lists, statistics, resident rows and
+    outputs, step after step, with one block per head and with several, with hits and with misses."""
+    decode, kernel = env
+    from spotlight_amd import _lib
+    L = _lib.load()
+    dtype = torch.bfloat16
+    B, QH, KH = 3, 16, 4
+    n_cap = (n0 + 32 + 7) // 8 * 8
+    try:
+        _lib.check(L.sl_tune(b"fused_rows", rows), "sl_tune")
+        inside, own = (_make_state(decode, _gen(70), B, QH, KH, n0, n_cap, k, dtype, lru=C, codes_layout="head") for _ in range(2))
+        g = _gen(71)
+        for step in range(6):
+            q = torch.randn(B, QH, 128, generator=g).to(dtype).to(DEV)
+            if step % 2 == 1:
+                q = prev_q          # the same query again: most selected rows are hits
+            prev_q = q
+            kn = torch.randn(B, KH, 128, generator=g).to(dtype).to(DEV)
+            vn = torch.randn(B, KH, 128, generator=g).to(dtype).to(DEV)
+            _lib.check(L.sl_tune(b"fused_lru", 1), "sl_tune")
+            a = inside.step(q, kn, vn).clone()
+            _lib.check(L.sl_tune(b"fused_lru", 0), "sl_tune")
+            b = own.step(q, kn, vn).clone()
+            assert not inside.peer_wait_failed() and not own.peer_wait_failed()
+            for name in ("idx", "slots_out", "slot_token", "slot_stamp", "token_slot", "lru_stats", "k_res", "v_res"):
+                assert torch.equal(getattr(inside, name), getattr(own, name)), (step, name)
+            assert torch.equal(a, b), step
+        stats = inside.lru_stats.cpu().numpy()
+        assert stats[..., 0].sum() > 0 and stats[..., 1].sum() > 0
+    finally:
+        _lib.check(L.sl_tune(b"fused_lru", 1), "sl_tune")
+        _lib.check(L.sl_tune(b"fused_rows", 0), "sl_tune")
+
+
 @pytest.mark.parametrize("B,QH,KH,n0,k,dtype,kind", DECODE_CASES[:4])
 def test_decode_step_two_launch_tail_matches_oracle(env, B, QH, KH, n0, k, dtype, kind):
     """The same step with selection and attention kept as two launches."""
