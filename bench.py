@@ -105,7 +105,7 @@ def main():
     tokens_timed = max(8, round(steps / L))
     tokens_warm = max(1, math.ceil(warmup / L))
     steps_timed, steps_warm = tokens_timed * L, tokens_warm * L
-    tokens = tokens_warm + tokens_timed + 4 + 64   # cache growth incl. the breakdown passes
+    tokens = tokens_warm + tokens_timed + 4 + 64 + 8   # cache growth incl. the cold tokens and the breakdown passes
     n_cap = (n0 + tokens + 7) // 8 * 8
     if args.floor_only:
         blocks = (n_cap + 4095) // 4096
@@ -186,10 +186,26 @@ def main():
     failed = [i for i, st in enumerate(layers) if st.peer_wait_failed()]
     if failed:
         raise RuntimeError(f"bounded peer wait ran out in layers {failed}: the timed steps are invalid")
+    # cold figure per token: a 1 GiB fill before each replay pushes the step's weights, codes and rows out
+    # of the L2s and the 256 MB memory-side cache -- what the model's own layers do between two decode
+    # steps of a layer (Llama-3-8B streams 0.4 GB of weights per layer); the timed replays above revisit
+    # each layer's data after only L - 1 other layers of this path
+    flush = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+    cold = []
+    for i in range(8):
+        flush.fill_(float(i))
+        c0.record()
+        token_graph.replay()
+        c1.record()
+        torch.cuda.synchronize()
+        cold.append(c0.elapsed_time(c1) * 1e3 / L)
+    del flush
+    cold.sort()
+    cold_token_us = cold[len(cold) // 2]
     n_mid = n0 + tokens_warm + tokens_timed / 2
     ab = algorithmic_bytes(c, n_mid)
     for st in layers:   # the graph advanced the lengths on the device; keep the host-side bound in step
-        st.host_len = n0 + tokens_warm + tokens_timed
+        st.host_len = n0 + tokens_warm + tokens_timed + 8
 
     if args.calibration_copy:
         src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
@@ -292,7 +308,7 @@ def main():
         "gpu_event_ms_per_step": round(gpu_ms / steps_timed, 6),
         "us_per_step_median_token": round(per_token_us[len(per_token_us) // 2], 3),
         "us_per_step_min_token": round(per_token_us[0], 3), "us_per_step_max_token": round(per_token_us[-1], 3),
-        "cold_first_token_us": round(cold_first_token_us, 3),
+        "cold_first_token_us": round(cold_first_token_us, 3), "cold_token_us": round(cold_token_us, 3),
         "lru_hit_rate": round(lru_hit_rate, 4) if lru_hit_rate is not None else None,
         "lru_miss_row_gbps": round(link_gbps, 1) if link_gbps is not None else None,
         "query_reuse": args.reuse,

@@ -84,7 +84,8 @@ __global__ __launch_bounds__(FS_THREADS) void score_select_attend_kernel(fused_a
 #pragma unroll
     for (int j = 0; j < FS_SLOTS; ++j) {
         const int64_t t = t_base + j * 64;
-        kreg[j] = kb[t < sa.n ? t : sa.n - 1];
+        const sl_u32x4 kv_ = __builtin_nontemporal_load(reinterpret_cast<const sl_u32x4 *>(kb + (t < sa.n ? t : sa.n - 1)));
+        kreg[j] = make_uint4(kv_.x, kv_.y, kv_.z, kv_.w);
     }
     int64_t n_b;
     int k_eff;

@@ -17,6 +17,25 @@
 
 namespace {
 
+// key codes are read once per step: streaming (non-temporal) loads
+template <int W>
+__device__ __forceinline__ void load_code_nt(const uint32_t *p, uint32_t (&c)[W]) {
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    if constexpr (W == 1) {
+        c[0] = __builtin_nontemporal_load(p);
+    } else if constexpr (W == 2) {
+        const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p));
+        c[0] = v.x; c[1] = v.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < W / 4; ++i) {
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p) + i);
+            c[4 * i] = v.x; c[4 * i + 1] = v.y; c[4 * i + 2] = v.z; c[4 * i + 3] = v.w;
+        }
+    }
+}
+
 template <int W>
 __device__ __forceinline__ void load_code(const uint32_t *p, uint32_t (&c)[W]) {
     if constexpr (W == 1) {
@@ -72,7 +91,7 @@ __global__ __launch_bounds__(HS_THREADS) void hamming_kernel(hamming_args a) {
 #pragma unroll
     for (int u = 0; u < HS_U; ++u) {
         const int64_t t = t0 + static_cast<int64_t>(u) * tok_per_pass + tl;
-        load_code<W>(kb + ((t < a.n ? t : a.n - 1) * KH + h) * W, kreg[u]);  // a.n rows exist whatever the length is
+        load_code_nt<W>(kb + ((t < a.n ? t : a.n - 1) * KH + h) * W, kreg[u]);  // a.n rows exist whatever the length is
     }
     // the sequence length is only needed from here on: it is read from memory, and
     // nothing above had to wait for it

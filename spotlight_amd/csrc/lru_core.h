@@ -298,8 +298,9 @@ __device__ __forceinline__ void lru_update(const lru_args &a, int b, int h, lru_
 #pragma unroll
                 for (int u = 0; u < LRU_CP; ++u)
                     if (dsts[u] >= 0) {
-                        *reinterpret_cast<u32x4 *>(kr + dsts[u]) = kbuf[u];
-                        *reinterpret_cast<u32x4 *>(vr + dsts[u]) = vbuf[u];
+                        // (streaming stores: the copied rows do not stay behind as dirty lines for the end of the launch)
+                        __builtin_nontemporal_store(kbuf[u], reinterpret_cast<u32x4 *>(kr + dsts[u]));
+                        __builtin_nontemporal_store(vbuf[u], reinterpret_cast<u32x4 *>(vr + dsts[u]));
                     }
             };
             issue(0);
