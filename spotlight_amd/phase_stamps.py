@@ -73,6 +73,8 @@ def main():
     ap.add_argument("--tokens", type=int, default=4)
     ap.add_argument("--codes-layout", default="auto")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE")
+    ap.add_argument("--cold", action="store_true",
+                    help="fill 1 GiB before the stamped token, so that its data (with --layers 1 also its code) come from HBM")
     args = ap.parse_args()
     import torch
 
@@ -108,11 +110,13 @@ def main():
         for st, (q, k, v) in zip(layers, ins):
             st.q_in.copy_(q); st.k_in.copy_(k); st.v_in.copy_(v)
             st._launch(n_max)
-    for _ in range(args.tokens):
+    for i in range(args.tokens):
+        if args.cold and i == args.tokens - 1:
+            torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
         graph.replay()
     torch.cuda.synchronize()
     print(f"config {args.config}: batch {B}, {c['n0']} rows, k = {c['k']}, codes {layers[0].codes_layout}-major, "
-          f"{L} layers rotated; stamps of the last layer's launches of the last token")
+          f"{L} layers rotated; stamps of the last layer's launches of the last token" + (", caches flushed before it" if args.cold else ""))
     for name in ("hash", "fused", "lru", "attn", "select_attend"):
         buf = read(lib, name)
         if buf is not None:
