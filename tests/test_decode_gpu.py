@@ -299,7 +299,7 @@ def test_decode_with_lru_gives_identical_attention(env, fuse, layout):
 
 
 @pytest.mark.parametrize("n0,k,C,rows", [(700, 30, 64, 0), (9000, 150, 1024, 3072), (9000, 150, 2048, 0), (20000, 300, 512, 4096),
-                                         (9000, 150, 4096, 0)])
+                                         (9000, 150, 4096, 0), (3000, 63, 64, 0), (5000, 2047, 2048, 0)])
 def test_table_update_inside_the_selection_launch_equals_the_launch_of_its_own(env, n0, k, C, rows):
     """Over head-major codes the block of a (b, kv head) that finishes last runs the head's table update
     at the end of the scorer + selection launch (tables of up to 2048 slots; larger ones keep the launch
