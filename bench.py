@@ -475,7 +475,7 @@ def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False, lru_inside=Fa
     B, QH, KH = c["B"], c["QH"], c["KH"]
     hash_rows = 1
     while hash_rows < 4 and (QH + KH) * ((B + hash_rows - 1) // hash_rows) > 256:
-        hash_rows *= 2
+        hash_rows += 1
     blocks4k = (n_max + 4095) // 4096
     grids = [((QH + KH) * ((B + hash_rows - 1) // hash_rows), 512),
              (((n_max * KH + 2047) // 2048) * B, 512)]

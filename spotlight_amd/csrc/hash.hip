@@ -101,7 +101,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     const int side_i = (a.n_sides > 1 && hh >= a.side[0].H) ? 1 : 0;
     const hash_side &sd = a.side[side_i];
     const int h = hh - (side_i ? a.side[0].H : 0);
-    static_assert(R == 1 || R == 2 || R == HK_B_PER_WG, "rows per workgroup");
+    static_assert(R >= 1 && R <= HK_B_PER_WG, "rows per workgroup");
     const int b_lo = blockIdx.y * R;
     const int b_hi = b_lo + R < a.B ? b_lo + R : a.B;
 
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     }
 }
 
-int g_hash_rows = 0;  // sl_tune("hash_rows", 0 | 1 | 2 | 4): batch rows per workgroup, 0 = by batch size
+int g_hash_rows = 0;  // sl_tune("hash_rows", 0 .. 4): batch rows per workgroup, 0 = by batch size
 
 template <typename T, int NL, int D_HID>
 int launch3(const hash_args &a, int Htot, hipStream_t s) {
@@ -335,11 +335,12 @@ int launch3(const hash_args &a, int Htot, hipStream_t s) {
     // its own (256 of them); rows taken together share barriers and weights but each
     // adds to the workgroup's critical path.
     int rows = 1;
-    while (rows < HK_B_PER_WG && static_cast<int64_t>(Htot) * ((a.B + rows - 1) / rows) > 256) rows *= 2;
+    while (rows < HK_B_PER_WG && static_cast<int64_t>(Htot) * ((a.B + rows - 1) / rows) > 256) ++rows;
     if (g_hash_rows && a.B > 1) rows = g_hash_rows;
     const dim3 grid(Htot, (a.B + rows - 1) / rows);
     if (rows == 1) hash_kernel<T, NL, D_HID, 1><<<grid, dim3(HK_THREADS), 0, s>>>(a);
     else if (rows == 2) hash_kernel<T, NL, D_HID, 2><<<grid, dim3(HK_THREADS), 0, s>>>(a);
+    else if (rows == 3) hash_kernel<T, NL, D_HID, 3><<<grid, dim3(HK_THREADS), 0, s>>>(a);
     else hash_kernel<T, NL, D_HID, HK_B_PER_WG><<<grid, dim3(HK_THREADS), 0, s>>>(a);
     return sl_check_launch();
 }
@@ -363,7 +364,7 @@ int launch(const hash_args &a, int Htot, hipStream_t s) {
 }  // namespace
 
 int sl_hash_tune(const char *key, int value) {
-    if (!strcmp(key, "hash_rows") && (value == 0 || value == 1 || value == 2 || value == 4)) { g_hash_rows = value; return SL_OK; }
+    if (!strcmp(key, "hash_rows") && (value >= 0 && value <= 4)) { g_hash_rows = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
 
