@@ -473,9 +473,9 @@ def latency_floor(dev, c, L, n_max, reps=8, one_launch_tail=False, lru_inside=Fa
     from spotlight_amd import _lib
     lib = _lib.load()
     B, QH, KH = c["B"], c["QH"], c["KH"]
-    hash_rows = 1
-    while hash_rows < 4 and (QH + KH) * ((B + hash_rows - 1) // hash_rows) > 256:
-        hash_rows += 1
+    # the library's rule: the fewest batch rows per hash workgroup (1, 2, 3, 4, 6, 8) that give one round of
+    # workgroups over the 256 compute units, else 4
+    hash_rows = next((r for r in (1, 2, 3, 4, 6, 8) if (QH + KH) * ((B + r - 1) // r) <= 256), 4)
     blocks4k = (n_max + 4095) // 4096
     grids = [((QH + KH) * ((B + hash_rows - 1) // hash_rows), 512),
              (((n_max * KH + 2047) // 2048) * B, 512)]

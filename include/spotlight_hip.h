@@ -54,7 +54,7 @@ int sl_version(void);
  * attention as one launch when the shapes allow and every 4096-token block keeps
  * at most 128 rows on average, 2 whenever the shapes allow, 0 never;
  * "hash_rows": batch rows one hash workgroup takes through the projections together
- * (1 to 4; 0 = by batch size, the default);
+ * (1, 2, 3, 4, 6 or 8; 0 = by batch size, the default);
  * "attn_wide_rows": rows per run from which the attention launch uses 8 waves per
  * workgroup instead of 4 (default 128);
  * "attn_mfma": 1 puts the q.K products of the attention on the matrix cores

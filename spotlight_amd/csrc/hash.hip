@@ -34,7 +34,7 @@ namespace {
 constexpr int HK_THREADS = 512;
 constexpr int HK_DIN = 128;
 constexpr int HK_NBITS = 128;
-constexpr int HK_B_PER_WG = 4;  // batch rows one workgroup takes when the batch is larger than one
+constexpr int HK_B_PER_WG = 8;  // most batch rows one workgroup takes through the projections together
 constexpr int HK_FOLD = 8;      // rows of a partial-sum table one lane folds in the first step
 
 __device__ __forceinline__ bool sl_aligned_dev(const void *p, uintptr_t a) {
@@ -79,7 +79,7 @@ __device__ __forceinline__ void fold_columns(const float *red, float *sub, float
 }
 
 // One workgroup of HK_THREADS lanes hashes head blockIdx.x (numbered over both
-// sides) for the batch rows [blockIdx.y * R, ..): R = 1 or HK_B_PER_WG rows go
+// sides) for the batch rows [blockIdx.y * R, ..): R rows go
 // through the projections TOGETHER, sharing every barrier and the weights in
 // registers (rows beyond the batch repeat the first row and store nothing).
 template <typename T, int NL, int D_HID, int R>
@@ -109,22 +109,18 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     // its batch rows first (they are needed first), then the weights of both
     // projections, the biases and the K / V rows the launch appends
     const T *xh = static_cast<const T *>(sd.x) + static_cast<int64_t>(h) * HK_DIN;
-    // (named scalars, picked by the loop counter below: an indexed array would not stay in registers)
-    static_assert(HK_B_PER_WG == 4, "four named input registers");
+    // (arrays indexed by fully unrolled loops only: they stay in registers)
     const T *xlane = xh + (tid & (HK_DIN - 1));
     const int nb = b_hi - b_lo;
-    const float x0 = to_f32(xlane[static_cast<int64_t>(b_lo) * sd.x_stride_b]);
-    const float x1 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 1 ? 1 : 0)) * sd.x_stride_b]);
-    const float x2 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 2 ? 2 : 0)) * sd.x_stride_b]);
-    const float x3 = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > 3 ? 3 : 0)) * sd.x_stride_b]);
+    float xrow[R], yrow[R];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) xrow[rr] = to_f32(xlane[static_cast<int64_t>(b_lo + (nb > rr ? rr : 0)) * sd.x_stride_b]);
     // rotary embedding: the partner element (i +- d/2), the frequency and the positions, loaded
     // whether or not they are used (without rope they re-read what is loaded anyway)
     const bool rope = a.rope_inv_freq != nullptr;
     const T *xpart = xh + ((tid + HK_DIN / 2) & (HK_DIN - 1));
-    const float y0 = to_f32(xpart[static_cast<int64_t>(b_lo) * sd.x_stride_b]);
-    const float y1 = to_f32(xpart[static_cast<int64_t>(b_lo + (nb > 1 ? 1 : 0)) * sd.x_stride_b]);
-    const float y2 = to_f32(xpart[static_cast<int64_t>(b_lo + (nb > 2 ? 2 : 0)) * sd.x_stride_b]);
-    const float y3 = to_f32(xpart[static_cast<int64_t>(b_lo + (nb > 3 ? 3 : 0)) * sd.x_stride_b]);
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) yrow[rr] = to_f32(xpart[static_cast<int64_t>(b_lo + (nb > rr ? rr : 0)) * sd.x_stride_b]);
     const float inv_freq = rope ? a.rope_inv_freq[tid & (HK_DIN / 2 - 1)] : 0.f;
     const int cg = tid % S1::LPR, r = tid / S1::LPR;
     float w1r[S1::PASSES][8];
@@ -146,22 +142,19 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     const T *b1p = sd.b1 ? static_cast<const T *>(sd.b1) + static_cast<int64_t>(h) * D_HID + (tid < D_HID ? tid : 0) : xh;
     const T *b2p = (NL == 2 && sd.b2) ? static_cast<const T *>(sd.b2) + static_cast<int64_t>(h) * HK_NBITS + (tid & (HK_NBITS - 1)) : xh;
     const float bias1 = to_f32(*b1p), bias2 = to_f32(*b2p);
-    // appended rows: (b_hi - b_lo) * CH <= 128 chunks of 16 bytes per tensor, one per lane
+    // appended rows: (b_hi - b_lo) * CH <= 256 chunks of 16 bytes per tensor, one per lane
     constexpr int CH = HK_DIN * sizeof(T) / 16;
     const bool cp_live = tid < (b_hi - b_lo) * CH;
     const int cp_b = b_lo + (cp_live ? tid / CH : 0), cp_c = cp_live ? tid % CH : 0;
     // destination rows of the batch rows (and of the lane's chunk of the appended rows)
     const int32_t *rowp = sd.code_row ? sd.code_row : reinterpret_cast<const int32_t *>(sd.codes);
-    const int32_t row0 = rowp[sd.code_row ? b_lo : 0];
-    const int32_t row1 = rowp[sd.code_row ? b_lo + (nb > 1 ? 1 : 0) : 0];
-    const int32_t row2 = rowp[sd.code_row ? b_lo + (nb > 2 ? 2 : 0) : 0];
-    const int32_t row3 = rowp[sd.code_row ? b_lo + (nb > 3 ? 3 : 0) : 0];
+    int32_t drow[R], prow[R];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) drow[rr] = rowp[sd.code_row ? b_lo + (nb > rr ? rr : 0) : 0];
     const int32_t cp_row = rowp[sd.code_row ? cp_b : 0];
     const int32_t *posp = rope ? a.rope_pos : rowp;
-    const int32_t pos0 = posp[rope ? b_lo : 0];
-    const int32_t pos1 = posp[rope ? b_lo + (nb > 1 ? 1 : 0) : 0];
-    const int32_t pos2 = posp[rope ? b_lo + (nb > 2 ? 2 : 0) : 0];
-    const int32_t pos3 = posp[rope ? b_lo + (nb > 3 ? 3 : 0) : 0];
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) prow[rr] = posp[rope ? b_lo + (nb > rr ? rr : 0) : 0];
     const T *src0 = sd.copy_src[0] ? static_cast<const T *>(sd.copy_src[0]) : static_cast<const T *>(sd.x);
     const T *src1 = sd.copy_src[1] ? static_cast<const T *>(sd.copy_src[1]) : static_cast<const T *>(sd.x);
     const int64_t cp_off = static_cast<int64_t>(cp_b) * sd.x_stride_b + h * HK_DIN;
@@ -184,13 +177,9 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
         }
     }
 
-    float xrow[4] = {x0, x1, x2, x3};
-    const int32_t drow[4] = {row0, row1, row2, row3};
     if (rope) {
         // out[i] = x[i] * cos + rot[i] * sin, rot = (-x[d/2:], x[:d/2]); cos / sin and every
         // product are rounded to T where the torch expression of the reference rounds them
-        const float yrow[4] = {y0, y1, y2, y3};
-        const int32_t prow[4] = {pos0, pos1, pos2, pos3};
         const float sgn = (tid & (HK_DIN / 2)) ? 1.f : -1.f;
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
@@ -211,7 +200,10 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     }
     // the step's row count per batch entry, for the launches that follow (head 0 of the last side)
     if (a.len_out && sd.code_row && side_i == a.n_sides - 1 && h == 0 && tid < nb) {
-        const int32_t n_now = (tid == 0 ? row0 : tid == 1 ? row1 : tid == 2 ? row2 : row3) + 1;
+        int32_t n_now = drow[0];
+#pragma unroll
+        for (int rr = 1; rr < R; ++rr) n_now = tid == rr ? drow[rr] : n_now;
+        n_now += 1;
         a.len_out[b_lo + tid] = n_now;
         if (a.keep_out) {
             const int32_t dropped = static_cast<int32_t>(static_cast<double>(n_now) * a.keep_mask_out);
@@ -327,21 +319,35 @@ __global__ __launch_bounds__(HK_THREADS) void hash_kernel(hash_args a) {
     }
 }
 
-int g_hash_rows = 0;  // sl_tune("hash_rows", 0 .. 4): batch rows per workgroup, 0 = by batch size
+int g_hash_rows = 0;  // sl_tune("hash_rows", 0 | 1 | 2 | 3 | 4 | 6 | 8): batch rows per workgroup, 0 = by batch size
 
 template <typename T, int NL, int D_HID>
 int launch3(const hash_args &a, int Htot, hipStream_t s) {
     // Rows per workgroup: the fewest that still give every workgroup a compute unit of
     // its own (256 of them); rows taken together share barriers and weights but each
-    // adds to the workgroup's critical path.
-    int rows = 1;
-    while (rows < HK_B_PER_WG && static_cast<int64_t>(Htot) * ((a.B + rows - 1) / rows) > 256) ++rows;
-    if (g_hash_rows && a.B > 1) rows = g_hash_rows;
+    // adds to the workgroup's critical path (alone: 4.4 us with one row, 9.3 with four, 12.2 with
+    // six, 14.5 with eight).  One round of workgroups beats more rounds of lighter ones while it can
+    // be had (batch 32 x 40 heads: 240 workgroups of six rows 12.8 us, 320 of four 15.9; batch 48:
+    // eight rows 15.1, four 16.4); beyond that four rows per workgroup measured best (batch 64: 22.8
+    // us, six rows 23.4, eight 27.5).
+    constexpr int MOST = D_HID > 256 ? 6 : 8;   // (the partial-sum tables of 8 rows of 512 hidden columns exceed the LDS)
+    static const int choices[] = {1, 2, 3, 4, 6, 8};
+    int rows = 0;
+    for (int c : choices)
+        if (rows == 0 && c <= MOST && static_cast<int64_t>(Htot) * ((a.B + c - 1) / c) <= 256) rows = c;
+    if (rows == 0) rows = 4;
+    if (g_hash_rows && a.B > 1 && g_hash_rows <= MOST) rows = g_hash_rows;
     const dim3 grid(Htot, (a.B + rows - 1) / rows);
-    if (rows == 1) hash_kernel<T, NL, D_HID, 1><<<grid, dim3(HK_THREADS), 0, s>>>(a);
-    else if (rows == 2) hash_kernel<T, NL, D_HID, 2><<<grid, dim3(HK_THREADS), 0, s>>>(a);
-    else if (rows == 3) hash_kernel<T, NL, D_HID, 3><<<grid, dim3(HK_THREADS), 0, s>>>(a);
-    else hash_kernel<T, NL, D_HID, HK_B_PER_WG><<<grid, dim3(HK_THREADS), 0, s>>>(a);
+    switch (rows) {
+        case 1: hash_kernel<T, NL, D_HID, 1><<<grid, dim3(HK_THREADS), 0, s>>>(a); break;
+        case 2: hash_kernel<T, NL, D_HID, 2><<<grid, dim3(HK_THREADS), 0, s>>>(a); break;
+        case 3: hash_kernel<T, NL, D_HID, 3><<<grid, dim3(HK_THREADS), 0, s>>>(a); break;
+        case 4: hash_kernel<T, NL, D_HID, 4><<<grid, dim3(HK_THREADS), 0, s>>>(a); break;
+        case 6: hash_kernel<T, NL, D_HID, 6><<<grid, dim3(HK_THREADS), 0, s>>>(a); break;
+        default:
+            if constexpr (MOST >= 8) hash_kernel<T, NL, D_HID, 8><<<grid, dim3(HK_THREADS), 0, s>>>(a);
+            else return SL_ERR_UNSUPPORTED;
+    }
     return sl_check_launch();
 }
 
@@ -364,7 +370,7 @@ int launch(const hash_args &a, int Htot, hipStream_t s) {
 }  // namespace
 
 int sl_hash_tune(const char *key, int value) {
-    if (!strcmp(key, "hash_rows") && (value >= 0 && value <= 4)) { g_hash_rows = value; return SL_OK; }
+    if (!strcmp(key, "hash_rows") && (value >= 0 && value <= 8 && value != 5 && value != 7)) { g_hash_rows = value; return SL_OK; }
     return SL_ERR_UNSUPPORTED;
 }
 

@@ -373,6 +373,38 @@ def test_hash_mlp_shipped_flavour_bf16_residue_and_biases(K, B, H):
     np.testing.assert_array_equal(rows[:, 0], got)
 
 
+@pytest.mark.parametrize("dims,dtype", [([128, 256, 128], torch.bfloat16), ([128, 128, 128], torch.float16), ([128, 512, 128], torch.bfloat16),
+                                        ([128, 128], torch.float32)])
+def test_hash_codes_do_not_depend_on_the_rows_a_workgroup_takes(K, dims, dtype):
+    """A workgroup of the hash launch takes 1 to 8 batch rows through the projections together; the
+    codes of a row must be the same bits whichever grouping ran, ragged last group included, and equal
+    the many-rows kernel's."""
+    from spotlight_amd import _lib
+    L = _lib.load()
+    g = _gen(77)
+    B, H = 13, 6
+    x = torch.randn(B, H, 128, generator=g).to(dtype).to(DEV)
+    layers = _hash_weights(g, H, dims, dtype, 0.08)
+    args = [t.to(DEV) for pair in layers for t in pair]
+    if len(layers) == 1:
+        args = [args[0], args[1], None, None]
+    want = None
+    try:
+        for rows in (1, 2, 3, 4, 6, 8):
+            if rows == 8 and dims[1] == 512:
+                continue   # no such flavour: its tables exceed the LDS
+            _lib.check(L.sl_tune(b"hash_rows", rows), "sl_tune")
+            got = K.hash_mlp_pack(x, args[0], args[1], args[2], args[3], residue=False).cpu().numpy()
+            if want is None:
+                want = got
+            np.testing.assert_array_equal(got, want, err_msg=f"{rows} rows per workgroup")
+    finally:
+        _lib.check(L.sl_tune(b"hash_rows", 0), "sl_tune")
+    if len(layers) == 2:
+        many = K.hash_rows_pack(x[:, None], args[0], args[1], args[2], args[3], False).cpu().numpy()
+        np.testing.assert_array_equal(many[:, 0], want)
+
+
 def test_hash_mlp_residue_and_no_bias(K):
     g = _gen(31)
     x = torch.randn(2, 8, 128, generator=g)
